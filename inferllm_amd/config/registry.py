@@ -44,9 +44,11 @@ def config_class(name: str) -> type:
 def config_from_dict(d: dict):
     """Typed configuration from the dict of a config.json."""
     archs = d.get("architectures")
+    if archs is None and isinstance(d.get("architecture"), str):
+        archs = [d["architecture"]]              # some designs name themselves with one string
     if not isinstance(archs, (list, tuple)) or len(archs) == 0 or not isinstance(archs[0], str):
-        raise ConfigError("config.json needs `architectures`: a list with the model class name; "
-                          f"registered: {registered_architectures()}")
+        raise ConfigError("config.json needs `architectures`: a list with the model class name "
+                          f"(or `architecture`: the name); registered: {registered_architectures()}")
     return config_class(archs[0]).from_dict(d)
 
 

@@ -28,12 +28,13 @@ class PartSpec:
 
 @dataclass
 class LayerSpec:
-    """A block: its arrangement ("pre_norm") and the parts it is made of."""
+    """A block: its arrangement ("pre_norm", "parallel") and the parts it is made of.  An
+    arrangement with one norm (both parts read its rows) has no `feed_forward_norm`."""
     block: str
     mixer: PartSpec
     feed_forward: PartSpec
     mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    feed_forward_norm: Optional[PartSpec] = None
     position: Optional[PartSpec] = None
 
 

@@ -15,6 +15,16 @@ int illm_version();
 // out[t, :] = table[tokens[t], :] as float32.
 int illm_embed(const int32_t* tokens, const void* table, int table_dt, float* out,
                int T, int E, int V, void* stream);
+// The same rows multiplied by `scale` (in float32).
+int illm_embed_scaled(const int32_t* tokens, const void* table, int table_dt, float* out,
+                      int T, int E, int V, float scale, void* stream);
+
+// out[i] = float32(a[i]) + float32(b[i]): the two outputs of a block whose parts read the same rows.
+int illm_sum_rows(const void* a, int a_dt, const void* b, int b_dt, float* out, size_t n,
+                  void* stream);
+
+// out[i] = max(x[i], 0)^2.
+int illm_relu_squared(const void* x, void* out, int dt, size_t n, void* stream);
 
 // Residual add and RMS norm.  in_row = row_idx ? row_idx[r] : r;
 // v = x[in_row] (+ delta[in_row]); when delta is given and row_idx is not, v is
@@ -204,6 +214,75 @@ int illm_sample_long_row_bytes(void);          // ILLM_SAMPLE_LONG_ROW_BYTES, fo
 int illm_sample_long(const float* logits, float* scratch, void* rows, int32_t* out, int B, int V,
                      float temp, float top_p, float repeat_penalty, const int32_t* last_tokens,
                      int n_last, const uint64_t* seeds, const int32_t* counters, void* stream);
+
+// ---- latent attention (csrc/latent_attention.hip).  A token keeps one normed latent row c [R] and one
+// rotated key part kr [dr] shared by all heads, together one row [R + dr] of the paged cache
+// [page][row in page][R + dr]; head h's key is [W_uk,h c | kr], its value W_uv,h c.
+//
+// Rows y [T, ncols] = [q: H (dn + dr) | down: R + dr | gate: H ...]: the first R of `down` are
+// RMS-normed (float32 statistics, weight norm_w, eps), the last dr and the last dr of every q head
+// are rotated in pairs (2i, 2i+1), i < rot/2, by cos_sin ([max_pos][rot/2][2] float32; null: no
+// rotation) at row_pos[t]; q is rotated in place; the normed latent and the rotated key part go
+// to the cache row of (row_slot[t], row_pos[t]) (null cache: nowhere) and to c_out [T, R] and
+// kr_out [T, dr] (either may be null).  slot_len, ring: as for illm_rope_store.
+int illm_latent_rope_store(void* y, int dt, int ncols, int T, int H, int dn, int dr, int R, int rot,
+                           const float* cos_sin, int max_pos, const void* norm_w, int norm_dt,
+                           float eps, const int32_t* row_pos, const int32_t* row_slot,
+                           const int32_t* slot_len, void* cache, const int32_t* page_table,
+                           int table_stride, int page_size, int ring, void* c_out, void* kr_out,
+                           void* stream);
+
+// Packed rows [q heads | k heads | v heads] with every head P wide (zeros beyond a head's own
+// dims) for the prompt attention kernels: q from y, keys [kvu's key part (dn) | kr (dr)], values
+// kvu's value part (dv); kvu [T, H dn + H dv] = c . [W_uk ; W_uv]^T.
+int illm_latent_pack(const void* y, int dt, int ncols, const void* kvu, const void* kr, void* out,
+                     int T, int H, int dn, int dr, int dv, int P, void* stream);
+
+// out[t, h dv + v] = attn[t, h P + v] * sigmoid(y[t, gate_off + h]).
+int illm_latent_gate(const void* attn, const void* y, int dt, int ncols, int gate_off, void* out,
+                     int T, int H, int dv, int P, void* stream);
+
+// qa[b, h] = [W_uk,h^T q_h (R) | rotated part of q_h (dr)] as float32 [B, H, R + dr], q from y.
+int illm_latent_absorb_q(const void* y, int dt, int ncols, const void* wuk, int w_dt, float* qa,
+                         int B, int H, int dn, int dr, int R, void* stream);
+
+// One token per sequence over the latent cache: scores qa[b, h] . cache row, softmax over the
+// keys the token sees (all, or the last `window`), sums of latent rows.  Token b sees
+// seq_len[b] + len_more keys, itself included.  partial: float32 [B][H][nsplit][R + 2] = (sums,
+// max, weight) per range of keys.  R <= 512.
+int illm_latent_attn_decode(const float* qa, const void* cache, int dt, const int32_t* page_table,
+                            int table_stride, int page_size, int ring, const int32_t* seq_slot,
+                            const int32_t* seq_len, int len_more, float* partial, int nsplit, int B,
+                            int H, int R, int dr, float scale, int window, void* stream);
+
+// out[b, h dv + v] = (W_uv[h dv + v, :] . combined sums of (b, h)) * sigmoid(y[b, gate_off + h]).
+int illm_latent_merge_up(const float* partial, int nsplit, const void* wuv, int w_dt, const void* y,
+                         int dt, int ncols, int gate_off, void* out, int B, int H, int R, int dv,
+                         void* stream);
+
+// ---- routed feed-forward (csrc/moe.hip).  Pair p = t * top + k is token t's k-th choice.
+// idx, wt [T, top]: the `top` outputs of z [T, NE] (float32) with the largest softmax(z) + corr
+// (corr may be null), in falling order, and their softmax values.  NE <= 512.
+int illm_moe_route(const float* z, const void* corr, int corr_dt, int T, int NE, int top,
+                   int32_t* idx, float* wt, void* stream);
+
+// order [NP]: the pairs whose choice is below NEr, grouped by choice; tiles [3 max_tiles + 1]:
+// (expert, first place in order, rows <= illm_moe_tile_rows()) per tile and, last, their number.
+// max_tiles >= min(NP, NP / tile rows + NEr).  NEr <= 512.
+int illm_moe_tile_rows(void);
+int illm_moe_group(const int32_t* idx, int NP, int NEr, int32_t* order, int32_t* tiles,
+                   int max_tiles, void* stream);
+
+// Y[p] = X[p / x_div] . W[e_p]^T for every grouped pair p (W [experts][N][K]); gated: W
+// [experts][2 N][K] = [gate | up] rows and Y[p] = silu(X Wg^T) * (X Wu^T).  Y [NP, N] of dt.
+int illm_moe_rows(const void* X, int x_div, const void* W, int dt, int gated, const int32_t* order,
+                  const int32_t* tiles, int max_tiles, void* Y, int N, int K, void* stream);
+
+// out[t] = sum_k wt[t, k] * (idx[t, k] < NEr ? Y[t top + k] : h[t]) (+ g * shared[t], with
+// g = sigmoid(h[t] . sg), or 1 if sg is null; shared may be null), float32 [T, E].
+int illm_moe_combine(const void* h, int dt, const int32_t* idx, const float* wt, const void* Y,
+                     const void* shared, const void* sg, int sg_dt, float* out, int T, int E, int top,
+                     int NEr, void* stream);
 
 #ifdef __cplusplus
 }

@@ -14,20 +14,58 @@
 
 // ---------------------------------------------------------------- embedding
 __global__ void embed_kernel(const int32_t* __restrict__ tokens, const void* __restrict__ table,
-                             int table_dt, float* __restrict__ out, int E, int V) {
+                             int table_dt, float* __restrict__ out, int E, int V, float scale) {
     const int t = blockIdx.x;
     int id = tokens[t];
     id = id < 0 ? 0 : (id >= V ? V - 1 : id);
     const size_t src = (size_t)id * E, dst = (size_t)t * E;
-    for (int i = threadIdx.x; i < E; i += blockDim.x) out[dst + i] = ld_f(table, table_dt, src + i);
+    for (int i = threadIdx.x; i < E; i += blockDim.x)
+        out[dst + i] = ld_f(table, table_dt, src + i) * scale;
+}
+
+extern "C" int illm_embed_scaled(const int32_t* tokens, const void* table, int table_dt, float* out,
+                                 int T, int E, int V, float scale, void* stream) {
+    if (T < 0 || E <= 0 || V <= 0 || !illm_dtype_ok(table_dt)) return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    hipLaunchKernelGGL(embed_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, tokens, table,
+                       table_dt, out, E, V, scale);
+    return illm_launch_status();
 }
 
 extern "C" int illm_embed(const int32_t* tokens, const void* table, int table_dt, float* out,
                           int T, int E, int V, void* stream) {
-    if (T < 0 || E <= 0 || V <= 0 || !illm_dtype_ok(table_dt)) return ILLM_ERR_ARG;
-    if (T == 0) return ILLM_OK;
-    hipLaunchKernelGGL(embed_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, tokens, table,
-                       table_dt, out, E, V);
+    return illm_embed_scaled(tokens, table, table_dt, out, T, E, V, 1.0f, stream);
+}
+
+// ---------------------------------------------------------------- sums and activations by element
+__global__ void sum_rows_kernel(const void* __restrict__ a, int a_dt, const void* __restrict__ b,
+                                int b_dt, float* __restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = ld_f(a, a_dt, i) + ld_f(b, b_dt, i);
+}
+
+extern "C" int illm_sum_rows(const void* a, int a_dt, const void* b, int b_dt, float* out,
+                             size_t n, void* stream) {
+    if (!illm_dtype_ok(a_dt) || !illm_dtype_ok(b_dt)) return ILLM_ERR_ARG;
+    if (n == 0) return ILLM_OK;
+    hipLaunchKernelGGL(sum_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, a, a_dt, b, b_dt, out, n);
+    return illm_launch_status();
+}
+
+__global__ void relu_squared_kernel(const void* __restrict__ x, void* __restrict__ out, int dt,
+                                    size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = fmaxf(ld_f(x, dt, i), 0.f);
+    st_f(out, dt, i, v * v);
+}
+
+extern "C" int illm_relu_squared(const void* x, void* out, int dt, size_t n, void* stream) {
+    if (!illm_dtype_ok(dt)) return ILLM_ERR_ARG;
+    if (n == 0) return ILLM_OK;
+    hipLaunchKernelGGL(relu_squared_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, x, out, dt, n);
     return illm_launch_status();
 }
 

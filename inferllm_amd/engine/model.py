@@ -37,7 +37,8 @@ class DecoderModel:
                 mixer=build_part("mixer", ls.mixer),
                 feed_forward=build_part("feed_forward", ls.feed_forward),
                 mixer_norm=build_part("norm", ls.mixer_norm),
-                feed_forward_norm=build_part("norm", ls.feed_forward_norm),
+                feed_forward_norm=(build_part("norm", ls.feed_forward_norm)
+                                   if ls.feed_forward_norm is not None else None),
                 position=position))
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)

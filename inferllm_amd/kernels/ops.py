@@ -96,15 +96,35 @@ def _check(rc: int, what: str) -> None:
 
 
 # ------------------------------------------------------------------ rows
-def embed(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """float32 [T, E] rows of `table` [V, E] at int32 `tokens` [T]."""
+def embed(tokens: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """float32 [T, E] rows of `table` [V, E] at int32 `tokens` [T], times `scale`."""
     _gpu(tokens, table)
     _i32(tokens)
     _need(table.dim() == 2 and tokens.dim() == 1, "embed: tokens [T], table [V, E]")
     T, (V, E) = tokens.numel(), table.shape
     out = torch.empty((T, E), dtype=torch.float32, device=table.device)
-    _check(_lib().illm_embed(_p(tokens), _p(table), _code(table), _p(out), T, E, V, _stream()),
-           "embed")
+    _check(_lib().illm_embed_scaled(_p(tokens), _p(table), _code(table), _p(out), T, E, V,
+                                    ctypes.c_float(scale), _stream()), "embed")
+    return out
+
+
+def sum_rows(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """float32(a) + float32(b), element by element: what a block whose mixer and feed-forward
+    read the same rows leaves for the residual stream."""
+    _gpu(a, b)
+    _need(a.shape == b.shape, f"sum_rows: {tuple(a.shape)} against {tuple(b.shape)}")
+    out = torch.empty(a.shape, dtype=torch.float32, device=a.device)
+    _check(_lib().illm_sum_rows(_p(a), _code(a), _p(b), _code(b), _p(out),
+                                ctypes.c_size_t(a.numel()), _stream()), "sum_rows")
+    return out
+
+
+def relu_squared(x: torch.Tensor) -> torch.Tensor:
+    """max(x, 0)^2, element by element."""
+    _gpu(x)
+    out = torch.empty_like(x)
+    _check(_lib().illm_relu_squared(_p(x), _p(out), _code(x), ctypes.c_size_t(x.numel()), _stream()),
+           "relu_squared")
     return out
 
 
@@ -1016,6 +1036,168 @@ def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
         _p(qkv), _p(out), _code(qkv), _p(kcache), _p(vcache), _p(page_table), page_table.shape[1],
         page_size, ring, _p(seq_slot), _p(seq_len), _p(partial), nsplit, B, nh, nkv, hd,
         ctypes.c_float(scale), window, _stream()), f"attn_decode (head_dim {hd})")
+    return out
+
+
+# ------------------------------------------------------------------ latent attention
+def latent_rope_store(y: torch.Tensor, H: int, dn: int, dr: int, R: int, rot: int,
+                      cos_sin: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
+                      row_pos: torch.Tensor, row_slot: torch.Tensor,
+                      slot_len: Optional[torch.Tensor], cache: Optional[torch.Tensor],
+                      page_table: Optional[torch.Tensor], page_size: int, ring: int,
+                      want_rows: bool):
+    """Rows y [T, >= H (dn + dr) + R + dr] = [q | down | ...]: the latent (first R of `down`) is
+    RMS-normed, the key part (last dr) and every q head's last dr dims are rotated (pairs
+    (2i, 2i+1), i < rot/2) at row_pos, q in place; latent and key part are stored in the paged
+    cache [pages, page_size, R + dr].  `want_rows`: also return them as (c [T, R], kr [T, dr])."""
+    _gpu(y, cos_sin, norm_w, row_pos, row_slot, slot_len, cache, page_table)
+    T, ncols = y.shape
+    _i32(row_pos, T); _i32(row_slot, T); _i32(slot_len); _i32(page_table)
+    _need(ncols >= H * (dn + dr) + R + dr, "latent_rope_store: rows too short")
+    _need(norm_w.shape == (R,), "latent_rope_store: norm weight [R]")
+    max_pos = 0
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.shape[1] * 2 == rot
+              and cos_sin.shape[2] == 2 and rot <= dr,
+              "latent_rope_store: angle table must be float32 [max_pos, rot/2, 2], rot <= dr")
+        max_pos = cos_sin.shape[0]
+    stride = 1
+    if cache is not None:
+        _need(cache.dtype == y.dtype and cache.dim() == 3 and cache.shape[1:] == (page_size, R + dr)
+              and page_table is not None and page_table.dim() == 2,
+              f"latent_rope_store: cache {tuple(cache.shape)} vs (pages, {page_size}, {R + dr})")
+        stride = page_table.shape[1]
+    c = torch.empty((T, R), dtype=y.dtype, device=y.device) if want_rows else None
+    kr = torch.empty((T, dr), dtype=y.dtype, device=y.device) if want_rows else None
+    _check(_lib().illm_latent_rope_store(
+        _p(y), _code(y), ncols, T, H, dn, dr, R, rot, _p(cos_sin), max_pos, _p(norm_w),
+        _code(norm_w), ctypes.c_float(eps), _p(row_pos), _p(row_slot), _p(slot_len), _p(cache),
+        _p(page_table), stride, page_size, ring, _p(c), _p(kr), _stream()), "latent_rope_store")
+    return c, kr
+
+
+def latent_pack(y: torch.Tensor, kvu: torch.Tensor, kr: torch.Tensor, H: int, dn: int, dr: int,
+                dv: int, P: int) -> torch.Tensor:
+    """Packed rows [q | k | v] of H heads, each P wide, for `attn_prefill`: q heads from y, key
+    heads [kvu's key part | kr], value heads from kvu's value part, zeros beyond a head's dims."""
+    _gpu(y, kvu, kr)
+    T = y.shape[0]
+    _need(kvu.shape == (T, H * (dn + dv)) and kr.shape == (T, dr) and kvu.dtype == y.dtype
+          and kr.dtype == y.dtype, "latent_pack: shapes or dtypes")
+    out = torch.empty((T, 3 * H * P), dtype=y.dtype, device=y.device)
+    _check(_lib().illm_latent_pack(_p(y), _code(y), y.shape[1], _p(kvu), _p(kr), _p(out), T, H, dn,
+                                   dr, dv, P, _stream()), "latent_pack")
+    return out
+
+
+def latent_gate(attn: torch.Tensor, y: torch.Tensor, gate_off: int, H: int, dv: int, P: int) -> torch.Tensor:
+    """[T, H dv]: the first dv dims of every head of attn [T, H P] times sigmoid(y[:, gate_off + h])."""
+    _gpu(attn, y)
+    T = y.shape[0]
+    _need(attn.shape == (T, H * P) and attn.dtype == y.dtype, "latent_gate: shapes or dtypes")
+    out = torch.empty((T, H * dv), dtype=y.dtype, device=y.device)
+    _check(_lib().illm_latent_gate(_p(attn), _p(y), _code(y), y.shape[1], gate_off, _p(out), T, H,
+                                   dv, P, _stream()), "latent_gate")
+    return out
+
+
+def latent_decode_splits(B: int, H: int, longest: int) -> int:
+    """Ranges the keys of a one-token step are cut into: about as many blocks as the chip has
+    compute units, at most 16 ranges, none shorter than 64 keys."""
+    groups = -(-H // (16 if H >= 16 else 8 if H >= 8 else 4))
+    return max(1, min(-(-256 // max(1, B * groups)), 16, (longest + 63) // 64))
+
+
+def latent_attn_decode(y: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor, gate_off: int,
+                       cache: torch.Tensor, page_table: torch.Tensor, page_size: int, ring: int,
+                       seq_slot: torch.Tensor, seq_len: torch.Tensor, len_more: int, H: int, dn: int,
+                       dr: int, R: int, dv: int, scale: float, window: int, nsplit: int) -> torch.Tensor:
+    """One token per sequence over the latent cache, never building a head's keys or values:
+    queries are taken through W_uk first, the weighted sums of latent rows through W_uv after,
+    then the head's output gate.  y [B, ...] = [q (rotated) | down | gate]; token b sees
+    seq_len[b] + len_more keys of the sequence in seq_slot[b], itself included; returns [B, H dv]."""
+    _gpu(y, w_uk, w_uv, cache, page_table, seq_slot, seq_len)
+    B = y.shape[0]
+    _i32(page_table); _i32(seq_slot, B); _i32(seq_len, B)
+    _need(w_uk.shape == (H * dn, R) and w_uv.shape == (H * dv, R), "latent_attn_decode: W_uk / W_uv")
+    _need(cache.dim() == 3 and cache.shape[1:] == (page_size, R + dr) and cache.dtype == y.dtype,
+          "latent_attn_decode: cache shape or dtype")
+    qa = torch.empty((B, H, R + dr), dtype=torch.float32, device=y.device)
+    _check(_lib().illm_latent_absorb_q(_p(y), _code(y), y.shape[1], _p(w_uk), _code(w_uk), _p(qa),
+                                       B, H, dn, dr, R, _stream()), "latent_absorb_q")
+    partial = torch.empty((B, H, nsplit, R + 2), dtype=torch.float32, device=y.device)
+    _check(_lib().illm_latent_attn_decode(
+        _p(qa), _p(cache), _code(cache), _p(page_table), page_table.shape[1], page_size, ring,
+        _p(seq_slot), _p(seq_len), len_more, _p(partial), nsplit, B, H, R, dr, ctypes.c_float(scale),
+        window, _stream()), f"latent_attn_decode (latent {R}+{dr})")
+    out = torch.empty((B, H * dv), dtype=y.dtype, device=y.device)
+    _check(_lib().illm_latent_merge_up(_p(partial), nsplit, _p(w_uv), _code(w_uv), _p(y), _code(y),
+                                       y.shape[1], gate_off, _p(out), B, H, R, dv, _stream()),
+           "latent_merge_up")
+    return out
+
+
+# ------------------------------------------------------------------ routed feed-forward
+def moe_route(z: torch.Tensor, correction: Optional[torch.Tensor], top: int):
+    """(idx int32 [T, top], weight float32 [T, top]): per row of the router's float32 outputs z
+    the `top` largest softmax(z) + correction, and their softmax values."""
+    _gpu(z, correction)
+    _need(z.dtype == torch.float32 and z.dim() == 2, "moe_route: float32 [T, outputs]")
+    T, NE = z.shape
+    _need(correction is None or correction.shape == (NE,), "moe_route: correction [outputs]")
+    idx = torch.empty((T, top), dtype=torch.int32, device=z.device)
+    wt = torch.empty((T, top), dtype=torch.float32, device=z.device)
+    _check(_lib().illm_moe_route(_p(z), _p(correction),
+                                 _code(correction) if correction is not None else 0, T, NE, top,
+                                 _p(idx), _p(wt), _stream()), "moe_route")
+    return idx, wt
+
+
+def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+    """Y [T * top, E]: for every (token, choice) pair whose choice is one of the stacked experts
+    (w_gate_up [experts, 2 F, E] = [gate | up], w_down [experts, E, F]) the expert's
+    down(silu(gate h) * (up h)); rows of other pairs are not written."""
+    _gpu(h, idx, w_gate_up, w_down)
+    _i32(idx)
+    T, E = h.shape
+    top = idx.shape[1]
+    n_exp, F2, _ = w_gate_up.shape
+    _need(w_gate_up.shape[2] == E and w_down.shape == (n_exp, E, F2 // 2) and F2 % 2 == 0
+          and w_gate_up.dtype == h.dtype and w_down.dtype == h.dtype and idx.shape[0] == T,
+          "moe_experts: shapes or dtypes")
+    NP = T * top
+    rows = _lib().illm_moe_tile_rows()
+    max_tiles = max(1, min(NP, NP // rows + n_exp))
+    order = torch.empty((NP,), dtype=torch.int32, device=h.device)
+    tiles = torch.empty((3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
+    _check(_lib().illm_moe_group(_p(idx), NP, n_exp, _p(order), _p(tiles), max_tiles, _stream()),
+           "moe_group")
+    act = torch.empty((NP, F2 // 2), dtype=h.dtype, device=h.device)
+    _check(_lib().illm_moe_rows(_p(h), top, _p(w_gate_up), _code(h), 1, _p(order), _p(tiles),
+                                max_tiles, _p(act), F2 // 2, E, _stream()), "moe_rows (gate|up)")
+    y = torch.empty((NP, E), dtype=h.dtype, device=h.device)
+    _check(_lib().illm_moe_rows(_p(act), 1, _p(w_down), _code(h), 0, _p(order), _p(tiles),
+                                max_tiles, _p(y), E, F2 // 2, _stream()), "moe_rows (down)")
+    return y
+
+
+def moe_combine(h: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor, y: Optional[torch.Tensor],
+                n_real: int, shared: Optional[torch.Tensor] = None,
+                shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [T, E]: sum over a token's choices of weight * (the expert's row of y, or h itself
+    for a choice >= n_real), plus sigmoid(h . shared_gate) * shared."""
+    _gpu(h, idx, wt, y, shared, shared_gate)
+    T, E = h.shape
+    top = idx.shape[1]
+    _need(y is not None or n_real == 0, "moe_combine: expert rows are needed")
+    _need(y is None or (y.shape == (T * top, E) and y.dtype == h.dtype), "moe_combine: expert rows")
+    _need(shared is None or (shared.shape == (T, E) and shared.dtype == h.dtype), "moe_combine: shared rows")
+    _need(shared_gate is None or shared_gate.numel() == E, "moe_combine: shared gate [E]")
+    out = torch.empty((T, E), dtype=torch.float32, device=h.device)
+    _check(_lib().illm_moe_combine(_p(h), _code(h), _p(idx), _p(wt), _p(y), _p(shared),
+                                   _p(shared_gate),
+                                   _code(shared_gate) if shared_gate is not None else 0, _p(out), T,
+                                   E, top, n_real, _stream()), "moe_combine")
     return out
 
 

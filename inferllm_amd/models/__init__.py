@@ -1,3 +1,3 @@
-from . import llama  # registers LlamaForCausalLM
+from . import llama, rabapel  # registers LlamaForCausalLM and Rabapel
 
-__all__ = ["llama"]
+__all__ = ["llama", "rabapel"]

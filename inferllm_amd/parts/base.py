@@ -189,15 +189,16 @@ class Block(Part):
     takes_prepared_rows = False
 
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
-                 feed_forward_norm: Norm, position: Optional[PositionEncoding]):
+                 feed_forward_norm: Optional[Norm], position: Optional[PositionEncoding]):
         super().__init__()
         self.mixer, self.feed_forward = mixer, feed_forward
         self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
         self.position = position
 
     def parts(self) -> List[Part]:
-        ps = [self.mixer, self.feed_forward, self.mixer_norm, self.feed_forward_norm]
-        return ps + ([self.position] if self.position is not None else [])
+        ps = [self.mixer, self.feed_forward, self.mixer_norm]
+        ps += [p for p in (self.feed_forward_norm, self.position) if p is not None]
+        return ps
 
     def wants(self) -> Dict[str, TensorWant]:
         out: Dict[str, TensorWant] = {}

@@ -44,3 +44,23 @@ class PreNormBlock(Block):
         if self.feed_forward.adds_residual:
             return self.feed_forward.forward(h2, ctx, residual=x, next_norm=next_norm)
         return self.feed_forward.forward(h2, ctx)
+
+
+@register_part("block", "parallel")
+class ParallelBlock(Block):
+    """x <- x + (mixer(h) + feed_forward(h)) with h = norm(x): one norm, both parts read its rows.
+
+    The two outputs are added in float32 and the sum is what the block leaves for the next norm
+    to add to the stream.  A feed-forward that returns None (a layer without one) leaves the
+    mixer's output alone.
+    """
+
+    graph_safe_prompts = True
+
+    def forward(self, x, pending, ctx: StepContext, line, writes_cache):
+        if isinstance(pending, ops.NormedRows):
+            pending = None                       # its sum is in x already
+        h = self.mixer_norm.forward(x, pending, ctx)
+        a = self.mixer.forward(h, ctx, line, writes_cache, self.position)
+        f = self.feed_forward.forward(h, ctx)
+        return a if f is None else ops.sum_rows(a, f)

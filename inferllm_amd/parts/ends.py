@@ -12,13 +12,15 @@ from .base import Embedding, Head, StepContext, register_part
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Embedding):
-    """Row copy, no scaling (src/kern/naive/naive.cpp:43-54); rows become float32."""
+    """Row copy (src/kern/naive/naive.cpp:43-54); rows become float32 and are multiplied by
+    `scale` (1: the reference's plain copy)."""
 
     graph_safe_prompts = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tensors=None):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, tensors=None):
         super().__init__(tensors)
         self.V, self.E = int(vocab_size), int(hidden_size)
+        self.scale = float(scale)
         self.weight: Optional[torch.Tensor] = None
 
     def shapes(self) -> Dict[str, TensorWant]:
@@ -28,7 +30,7 @@ class TokenEmbedding(Embedding):
         self.weight = self._take(tensors, "weight").contiguous()
 
     def forward(self, ctx: StepContext):
-        return ops.embed(ctx.tokens, self.weight)
+        return ops.embed(ctx.tokens, self.weight, self.scale)
 
 
 @register_part("head", "lm_head")
