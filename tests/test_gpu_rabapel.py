@@ -1,0 +1,269 @@
+"""Rabapel through the engine against the plain model (tests/plain_rabapel.py): whole prompts,
+token-by-token decoding, prompts cut into portions, batches of unequal requests, slots and pages
+used again, planted keys at window edges, page borders and far away, greedy generation; and the
+router and expert kernels alone.  Configurations: tests/rabapel_tiny.py."""
+import pytest
+import torch
+
+import plain_rabapel as P
+from rabapel_tiny import MIXED, ODD, plant_key, rel_err, single, weights64, write_model
+from tiny import random_ids
+
+pytestmark = pytest.mark.gpu
+
+BUDGET = {"float32": 2e-5, "bfloat16": 4e-2}
+STORE = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def engine_for(d, dtype, **kw):
+    import inferllm_amd as I
+    kw.setdefault("max_batch", 8)
+    kw.setdefault("max_seq_len", 1024)
+    kw.setdefault("poison_freed", True)
+    return I.Engine.from_pretrained(d, dtype=dtype, device="cuda:0", **kw)
+
+
+def feed(eng, slot, tokens, cuts):
+    """Logits of every position of `tokens`, fed in steps that end at `cuts` (then one by one)."""
+    from inferllm_amd import StepEntry
+    rows, at = [], 0
+    for c in list(cuts) + list(range((cuts[-1] if cuts else 0) + 1, len(tokens) + 1)):
+        if c <= at:
+            continue
+        rows.append(eng.step([StepEntry(slot, tokens[at:c], list(range(c - at)))]).clone())
+        at = c
+    return torch.cat(rows)
+
+
+def close(got, want, dtype, what=""):
+    """float32: every row within the budget.  bfloat16: rounding of the activations can turn a
+    router's close call, which moves one token's output; all rows but a few within the budget."""
+    scale = want.abs().max()
+    err = (got.double().cpu() - want).abs().amax(dim=-1) / scale
+    if dtype == "float32":
+        assert float(err.max()) < BUDGET[dtype], (what, float(err.max()))
+    else:
+        over = int((err > BUDGET[dtype]).sum())
+        assert over <= max(1, len(err) // 20) and float(err.median()) < BUDGET[dtype] / 2, \
+            (what, over, len(err), float(err.median()))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["MIXED", "ODD"])
+def test_whole_prompts_of_unequal_lengths_then_tokens(tmp_path_factory, name, dtype):
+    """Several prompts in one step (1 to 140 tokens, the first tokens of each included), then
+    four steps of one token each for all of them, against the plain model of each alone."""
+    from inferllm_amd import StepEntry
+    config = {"MIXED": MIXED, "ODD": ODD}[name]
+    d = write_model(tmp_path_factory.getbasetemp(), config, seed=3, dtype=STORE[dtype])
+    w = weights64(d)
+    eng = engine_for(d, dtype)
+    reqs = [random_ids(n + 4, config["vocab"], 11 * n) for n in (1, 2, 140, 65, 33, 71)]
+    slots = [eng.alloc_slot() for _ in reqs]
+    got = [[] for _ in reqs]
+    out = eng.step([StepEntry(s, r[:-4], list(range(len(r) - 4))) for s, r in zip(slots, reqs)])
+    at = 0
+    for i, r in enumerate(reqs):
+        got[i].append(out[at:at + len(r) - 4].clone())
+        at += len(r) - 4
+    for t in (4, 3, 2, 1):
+        out = eng.step([StepEntry(s, [r[-t]], [0]) for s, r in zip(slots, reqs)])
+        for i in range(len(reqs)):
+            got[i].append(out[i:i + 1].clone())
+    for i, r in enumerate(reqs):
+        close(torch.cat(got[i]), P.forward(config, w, r), dtype, f"request {i}")
+    for s in slots:
+        eng.free_slot(s)
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_past_windows_and_pages(tmp_path_factory, dtype):
+    """A prompt of 9 tokens, then 190 tokens one by one: the windows of 70 and 33 keys pass over
+    decoded tokens, pages of 64 fill up and the windows' rings of pages come round."""
+    d = write_model(tmp_path_factory.getbasetemp(), MIXED, seed=5, dtype=STORE[dtype])
+    w = weights64(d)
+    eng = engine_for(d, dtype, step_rows=16)
+    toks = random_ids(199, MIXED["vocab"], 1)
+    s = eng.alloc_slot()
+    close(feed(eng, s, toks, [9]), P.forward(MIXED, w, toks), dtype)
+    eng.free_slot(s)
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_portions_of_a_prompt(tmp_path_factory, graphs):
+    """A prompt fed in portions of 2 to 90 tokens (and single ones between) gives what the whole
+    prompt gives; the portions cross pages and are longer and shorter than the windows."""
+    d = write_model(tmp_path_factory.getbasetemp(), MIXED, seed=7)
+    w = weights64(d)
+    eng = engine_for(d, "float32", use_graphs=graphs)
+    toks = random_ids(230, MIXED["vocab"], 2)
+    want = P.forward(MIXED, w, toks)
+    for cuts in ([2, 4, 7, 71, 73, 163, 228], [64, 128, 129, 131, 221], [90, 92, 180, 230]):
+        s = eng.alloc_slot()
+        got = feed(eng, s, toks, cuts)
+        eng.free_slot(s)
+        assert rel_err(got, want) < BUDGET["float32"], cuts
+
+
+def test_a_request_alone_and_in_company(tmp_path_factory):
+    """The logits of a request do not depend on what else is in the batch beyond rounding, and
+    slots and pages that were freed (and filled with NaN) are used again."""
+    from inferllm_amd import StepEntry
+    d = write_model(tmp_path_factory.getbasetemp(), MIXED, seed=9)
+    eng = engine_for(d, "float32")
+    reqs = [random_ids(n, MIXED["vocab"], 7 * n) for n in (40, 141, 9, 90)]
+    alone = []
+    for r in reqs:
+        s = eng.alloc_slot()
+        alone.append(feed(eng, s, r, [len(r) - 6]))
+        eng.free_slot(s)
+    for order in ([0, 1, 2, 3], [3, 1, 0, 2]):
+        slots = {i: eng.alloc_slot() for i in order}
+        out = eng.step([StepEntry(slots[i], reqs[i][:-6], list(range(len(reqs[i]) - 6))) for i in order])
+        at, got = 0, {i: [] for i in order}
+        for i in order:
+            got[i].append(out[at:at + len(reqs[i]) - 6].clone())
+            at += len(reqs[i]) - 6
+        for t in range(6, 0, -1):
+            live = [i for i in order if not (i == 2 and t < 4)]      # one request ends earlier
+            if t == 3:
+                eng.free_slot(slots[2])
+            out = eng.step([StepEntry(slots[i], [reqs[i][-t]], [0]) for i in live])
+            for k, i in enumerate(live):
+                got[i].append(out[k:k + 1].clone())
+        for i in order:
+            g = torch.cat(got[i])
+            n = g.shape[0]
+            assert rel_err(g, alone[i][:n].double().cpu()) < 1e-5, (order, i)
+            if i != 2:
+                eng.free_slot(slots[i])
+    eng.cache.check()
+
+
+def _planted(tmp, window, mlp=None):
+    config = single(window=window, mlp=mlp)
+    A, B = 17, 23
+    d = write_model(tmp, config, seed=window or 1, edit=lambda w: plant_key(w, config, A, B))
+    return config, d, A, B
+
+
+def _sequence(config, A, B, at, gap, tail=0):
+    """Filler tokens with the planted key token at place `at` and the query token `gap` later."""
+    fill = [t for t in random_ids(at + gap + tail + 40, config["vocab"], at * 1000 + gap) if t not in (A, B)]
+    seq = fill[:at] + [A] + fill[at:at + gap - 1] + [B] + fill[at + gap - 1:at + gap - 1 + tail]
+    return seq
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_planted_key_just_inside_and_outside_the_window(tmp_path_factory, dtype):
+    """The query token's score for the key token stands out, so its logits turn on whether the
+    key is seen: at distance window - 1 it is, at distance window it is not.  Keys at the start
+    of a sequence, at page borders and in the middle; the query in a prompt and decoded alone."""
+    window = 70
+    config, d, A, B = _planted(tmp_path_factory.getbasetemp(), window)
+    if dtype == "bfloat16":
+        d = write_model(tmp_path_factory.getbasetemp(), config, seed=window, dtype=torch.bfloat16,
+                        edit=lambda w: plant_key(w, config, A, B))
+    w = weights64(d)
+    eng = engine_for(d, dtype)
+    for at in (0, 5, 63, 64, 100, 127):
+        rows = {}
+        for gap in (window - 1, window):
+            seq = _sequence(config, A, B, at, gap, tail=2)
+            want = P.forward(config, w, seq)
+            rows[gap] = want[at + gap]
+            for cut in (len(seq), at + gap):              # the query in the prompt / decoded alone
+                s = eng.alloc_slot()
+                got = feed(eng, s, seq, [cut])
+                eng.free_slot(s)
+                err = rel_err(got[at + gap - 1:], want[at + gap - 1:])
+                assert err < BUDGET[dtype], (at, gap, cut, err)
+        # the plant works: seen or not seen is a difference of the logits' own size
+        assert float((rows[window - 1] - rows[window]).abs().max() / rows[window].abs().max()) > 0.2
+
+
+def test_a_planted_key_far_away(tmp_path_factory):
+    """Without a window a key hundreds of tokens back, also on a page border, is still seen: the
+    plain model with that key masked differs by the logits' own size."""
+    config, d, A, B = _planted(tmp_path_factory.getbasetemp(), None,
+                               mlp={"kind": "dense", "ff": 100})
+    w = weights64(d)
+    eng = engine_for(d, "float32")
+    for at, gap in ((0, 300), (64, 257), (127, 400), (3, 511)):
+        seq = _sequence(config, A, B, at, gap, tail=1)
+        want = P.forward(config, w, seq)
+        for cut in (len(seq), at + gap, at + 2):
+            s = eng.alloc_slot()
+            got = feed(eng, s, seq, [cut] if cut > at + 2 else [cut, at + gap])
+            eng.free_slot(s)
+            assert rel_err(got[at + gap:], want[at + gap:]) < BUDGET["float32"], (at, gap, cut)
+        near = dict(config, layers=[dict(config["layers"][0],
+                                         mixer=dict(config["layers"][0]["mixer"], mask={"size": gap}))])
+        blind = P.forward(near, w, seq)[at + gap]
+        assert float((blind - want[at + gap]).abs().max() / want[at + gap].abs().max()) > 0.2
+
+
+def test_greedy_generation_through_the_engine(tmp_path_factory):
+    """`Engine.generate` (scheduler, sampler, decode graphs) gives the plain model's greedy tokens."""
+    d = write_model(tmp_path_factory.getbasetemp(), MIXED, seed=13)
+    w = weights64(d)
+    eng = engine_for(d, "float32")
+    prompts = [random_ids(n, MIXED["vocab"], 3 * n) for n in (5, 68, 1, 31)]
+    got = eng.generate(prompts, max_new_tokens=8, stop_token_ids=[])
+    assert got == [P.generate_greedy(MIXED, w, p, 8) for p in prompts]
+    assert eng.generate(prompts[:2], max_new_tokens=4, stop_token_ids=[], max_step_tokens=16) == \
+        [g[:4] for g in got[:2]]
+    eng.cache.check()
+
+
+def test_architecture_is_chosen_by_config_and_refuses_what_it_lacks(tmp_path_factory):
+    import inferllm_amd as I
+    assert "Rabapel" in I.registered_architectures()
+    bad = dict(MIXED, layers=[dict(MIXED["layers"][0], type="something_else")])
+    with pytest.raises(I.ConfigError):
+        I.config_from_dict(bad)
+
+
+# ---------------------------------------------------------------- mechanisms alone
+@pytest.mark.parametrize("n_out,top", [(7, 3), (16, 2), (130, 8), (3, 1)])
+def test_router_kernel(n_out, top):
+    from inferllm_amd.kernels import ops
+    g = torch.Generator().manual_seed(n_out)
+    z = torch.randn((50, n_out), generator=g) * 2
+    corr = torch.randn((n_out,), generator=g) * 0.3
+    idx, wt = ops.moe_route(z.cuda(), corr.cuda(), top)
+    s = torch.softmax(z.double(), -1)
+    want = torch.topk(s + corr.double(), top, dim=-1).indices
+    assert torch.equal(idx.cpu().long(), want)
+    assert float((wt.cpu().double() - torch.gather(s, 1, want)).abs().max()) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("E,F,n_real,n_id,top,T", [(64, 40, 5, 2, 3, 37), (90, 30, 2, 0, 1, 9),
+                                                   (128, 96, 12, 4, 2, 300)])
+def test_expert_kernels(dtype, E, F, n_real, n_id, top, T):
+    """Grouping, the experts' products and the weighted sum against a loop over tokens."""
+    from inferllm_amd.kernels import ops
+    g = torch.Generator().manual_seed(E + T)
+    h = torch.randn((T, E), generator=g).to(dtype)
+    wgu = (torch.randn((n_real, 2 * F, E), generator=g) * 0.2).to(dtype)
+    wd = (torch.randn((n_real, E, F), generator=g) * 0.2).to(dtype)
+    idx = torch.stack([torch.randperm(n_real + n_id, generator=g)[:top] for _ in range(T)]).to(torch.int32)
+    wt = torch.rand((T, top), generator=g)
+    shared = torch.randn((T, E), generator=g).to(dtype)
+    sg = torch.randn((E,), generator=g).to(dtype) * 0.1
+    y = ops.moe_experts(h.cuda(), idx.cuda(), wgu.cuda(), wd.cuda())
+    out = ops.moe_combine(h.cuda(), idx.cuda(), wt.cuda(), y, n_real, shared.cuda(), sg.cuda())
+    h64, want = h.double(), torch.zeros((T, E), dtype=torch.float64)
+    for t in range(T):
+        for k in range(top):
+            e = int(idx[t, k])
+            if e < n_real:
+                gu = wgu[e].double() @ h64[t]
+                v = wd[e].double() @ (torch.nn.functional.silu(gu[:F]) * gu[F:])
+            else:
+                v = h64[t]
+            want[t] += wt[t, k].double() * v
+        want[t] += torch.sigmoid(h64[t] @ sg.double()) * shared[t].double()
+    assert rel_err(out, want) < (1e-5 if dtype == torch.float32 else 2e-2)
