@@ -21,6 +21,11 @@ cache of its live sequences) / its time / the HBM peak.  Peaks are the published
 of MI355X (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, float32 157.3 TFLOP/s).
 The run fails (non-zero) if any timed run produced a non-finite logit or the same
 greedy token everywhere.
+
+`--design rabapel` is another workload with a line of its own (the default's stays as it is):
+Rabapel (latent attention, layers that alternate a dense and a routed feed-forward) at two
+sizes beside LLaMA at the same width, heads and layer count: prefill of 2,048 tokens and decoding
+at batch 1, 8 and 64, each with its fraction of the matrix or HBM peak.
 """
 import argparse
 import json
@@ -100,6 +105,22 @@ class Bench:
     def ids(self, n):
         return self.torch.randint(0, self.cfg["vocab_size"], (n,), generator=self.g).tolist()
 
+    @classmethod
+    def around(cls, eng, vocab, layers, dtype, step_bytes, flops, seed=1234):
+        """A bench around an engine that is there already (another design): `step_bytes(batch,
+        mean_ctx)` and `flops(tokens, lens)` are the design's own counts."""
+        import torch
+        b = cls.__new__(cls)
+        b.torch, b.eng, b.cfg, b.layers, b.full_layers = torch, eng, {"vocab_size": vocab}, layers, layers
+        b.esz = 2 if dtype == "bfloat16" else 4
+        b.dkey = "bf16" if dtype == "bfloat16" else "fp32"
+        b.g = torch.Generator().manual_seed(seed)
+        b.step_bytes = step_bytes
+        b.flops = flops
+        return b
+
+    flops = None
+
     def step_bytes(self, batch, mean_ctx):
         return (weight_bytes_per_step(self.cfg, self.layers, self.esz)
                 + batch * mean_ctx * kv_bytes_per_token(self.cfg, self.layers, self.esz))
@@ -162,7 +183,8 @@ class Bench:
             for s in slots:
                 eng.free_slot(s)
         pt = min(times[skip:])
-        fl = prefill_flops(self.cfg, self.layers, T * prompts, prompts, [T] * prompts)
+        fl = (self.flops(T * prompts, [T] * prompts) if self.flops is not None else
+              prefill_flops(self.cfg, self.layers, T * prompts, prompts, [T] * prompts))
         return {"value": round(T * prompts / pt, 1), "tokens": T * prompts, "ms": round(pt * 1e3, 3),
                 "frac": round(fl / pt / (PEAK_TFLOPS[self.dkey] * 1e12), 4)}
 
@@ -189,6 +211,113 @@ class Bench:
         return pf, pf_frac, B * steps / st.decode_seconds, frac
 
 
+# ---------------------------------------------------------------- another design beside LLaMA
+def rabapel_config(width, heads, layers, dense_ff, experts, expert_ff, top, shared_ff, vocab=32000,
+                   window=None):
+    """Layers that alternate a dense and a routed feed-forward; heads of 128 + 64 query dims,
+    128 value dims and a latent of 512, the sizes such heads have in published models."""
+    mixer = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
+             "rot": {"base": 10000.0, "dims": 64,
+                     "scaling": {"factor": 40.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    if window:
+        mixer["mask"] = {"size": window}
+    dense = {"kind": "dense", "ff": dense_ff}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff},
+           "router": {"experts": experts, "identity": 0, "top": top}, "shared": {"ff": shared_ff}}
+    return {"architecture": "Rabapel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "max_positions": 8192,
+            "layers": [{"type": "latent_attention", "mixer": dict(mixer), "mlp": moe if i % 2 else dense}
+                       for i in range(layers)]}
+
+
+def rabapel_counts(cfg, esz):
+    """(step_bytes(batch, mean_ctx), flops(tokens, lens)) of a Rabapel configuration: the weights
+    a decode step has to read (of a routed layer: router, shared expert and the experts that
+    `batch` tokens are expected to choose among them) and its cache rows; the multiply-adds of a
+    prompt step with every head's keys and values made from the latent rows."""
+    E, V = cfg["width"], cfg["vocab"]
+
+    def layer_parts(layer):
+        m, mlp = layer["mixer"], layer["mlp"]
+        H, dq, dv, R, dr = m["heads"], m["dim"] + m["rot_dim"], m["vdim"], m["kv_rank"], m["rot_dim"]
+        mix = E * (H * dq + R + dr + H) + R * H * (m["dim"] + dv) + E * H * dv
+        return m, mlp, mix
+
+    def step_bytes(batch, mean_ctx):
+        total = V * E
+        for layer in cfg["layers"]:
+            m, mlp, mix = layer_parts(layer)
+            total += mix + batch * min(mean_ctx, (m.get("mask") or {}).get("size") or mean_ctx) * (m["kv_rank"] + m["rot_dim"])
+            if mlp["kind"] == "dense":
+                total += 2 * E * mlp["ff"]
+            else:
+                n, top = mlp["router"]["experts"], mlp["router"]["top"]
+                used = n * (1.0 - (1.0 - top / n) ** batch)
+                total += E * n + 3 * E * mlp["shared"]["ff"] + used * 3 * E * mlp["expert"]["ff"]
+        return total * esz
+
+    def flops(tokens, lens):
+        total = 2.0 * len(lens) * V * E
+        for layer in cfg["layers"]:
+            m, mlp, mix = layer_parts(layer)
+            H, dq, dv = m["heads"], m["dim"] + m["rot_dim"], m["vdim"]
+            w = (m.get("mask") or {}).get("size")
+            pairs = sum(n * (n + 1) / 2 if not w or n <= w else w * (w + 1) / 2 + (n - w) * w for n in lens)
+            total += 2.0 * tokens * mix + 2.0 * H * (dq + dv) * pairs
+            if mlp["kind"] == "dense":
+                total += 2.0 * tokens * 2 * E * mlp["ff"]
+            else:
+                r = mlp["router"]
+                total += 2.0 * tokens * (E * r["experts"] + 3 * E * mlp["shared"]["ff"]
+                                         + r["top"] * 3 * E * mlp["expert"]["ff"])
+        return total
+
+    return step_bytes, flops
+
+
+def rabapel_main(args) -> int:
+    """Rabapel at two sizes beside LLaMA of the same width, heads and number of layers (four: the
+    figures are per design and size, tokens/s of these four-layer models, with the fraction of the
+    matrix peak for prompts and of the HBM peak for decode steps)."""
+    import torch
+    from inferllm_amd import Engine
+    layers = args.layers or 4
+    esz = 2 if args.dtype == "bfloat16" else 4
+    sizes = {"2048": dict(width=2048, heads=16, dense_ff=8192, experts=64, expert_ff=1408, top=6, shared_ff=2816),
+             "4096": dict(width=4096, heads=32, dense_ff=11008, experts=32, expert_ff=2048, top=4, shared_ff=4096)}
+    few = min(args.steps, 128)
+    out = {"metric": "Rabapel beside LLaMA at equal width, heads and layers: prefill tok/s at 2,048 tokens, decode tok/s at batch 1/8/64",
+           "unit": "tokens/s", "n_gpus": 1, "steps": few, "warmup": 4, "dtype": "bf16" if esz == 2 else "fp32",
+           "data": "synthetic: seeded random weights N(0, 0.02), uniform random token ids",
+           "layers": layers, "sizes": {}}
+    for name, sz in sizes.items():
+        if args.size and args.size != name:
+            continue
+        row = {}
+        rcfg = rabapel_config(layers=layers, **sz)
+        lcfg = dict(LLAMA2_7B, hidden_size=sz["width"], intermediate_size=sz["dense_ff"],
+                    num_attention_heads=sz["heads"], num_key_value_heads=sz["heads"],
+                    num_hidden_layers=layers, max_position_embeddings=8192)
+        for design in ("rabapel", "llama"):
+            if design == "rabapel":
+                eng = Engine.from_random(rcfg, seed=0, dtype=args.dtype, device="cuda:0", max_batch=64,
+                                         max_seq_len=4096, max_tokens=64 * 1024)
+                b = Bench.around(eng, rcfg["vocab"], layers, args.dtype, *rabapel_counts(rcfg, esz))
+            else:
+                b = Bench(lcfg, layers, args.dtype, 64, 64 * 1024)
+            torch.cuda.synchronize()
+            r = {"prefill_2048": b.prefill_run(2048, reps=4)}
+            for batch in (1, 8, 64):
+                v, ms, f = b.decode_run(batch, few, 4, args.prompt)
+                r[f"decode_b{batch}"] = {"value": round(v, 1), "ms": round(ms, 4), "hbm_frac": round(f, 4)}
+            row[design] = r
+            b.close()
+            del b
+        out["sizes"][name] = row
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -206,10 +335,16 @@ def main() -> int:
     ap.add_argument("--no-70b", action="store_true",
                     help="leave the LLaMA-2-70B shape out of `points` (138 GB of weights: half a minute)")
     ap.add_argument("--with-70b", action="store_true", help="(the default now; kept for old command lines)")
+    ap.add_argument("--design", default="llama", choices=["llama", "rabapel"],
+                    help="rabapel: that design at two sizes beside LLaMA at equal size (a line of its own)")
+    ap.add_argument("--size", default="", help="with --design rabapel: only this width (2048 or 4096)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only (this library has no multi-GPU path); --gpus must be 1")
         return 2
+
+    if args.design == "rabapel":
+        return rabapel_main(args)
 
     shape_name, shape_cfg = SHAPES[args.shape]
     ctx_len = shape_cfg["max_position_embeddings"]

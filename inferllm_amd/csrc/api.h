@@ -224,13 +224,15 @@ int illm_sample_long(const float* logits, float* scratch, void* rows, int32_t* o
 // are rotated in pairs (2i, 2i+1), i < rot/2, by cos_sin ([max_pos][rot/2][2] float32; null: no
 // rotation) at row_pos[t]; q is rotated in place; the normed latent and the rotated key part go
 // to the cache row of (row_slot[t], row_pos[t]) (null cache: nowhere) and to c_out [T, R] and
-// kr_out [T, dr] (either may be null).  slot_len, ring: as for illm_rope_store.
+// kr_out [T, dr] (either may be null).  slot_len, ring: as for illm_rope_store.  cache_t (may be
+// null): a second copy of the latent alone, laid out [page][R][row in page], for
+// illm_latent_attn_decode_mfma.
 int illm_latent_rope_store(void* y, int dt, int ncols, int T, int H, int dn, int dr, int R, int rot,
                            const float* cos_sin, int max_pos, const void* norm_w, int norm_dt,
                            float eps, const int32_t* row_pos, const int32_t* row_slot,
                            const int32_t* slot_len, void* cache, const int32_t* page_table,
                            int table_stride, int page_size, int ring, void* c_out, void* kr_out,
-                           void* stream);
+                           void* cache_t, void* stream);
 
 // Packed rows [q heads | k heads | v heads] with every head P wide (zeros beyond a head's own
 // dims) for the prompt attention kernels: q from y, keys [kvu's key part (dn) | kr (dr)], values
@@ -255,28 +257,47 @@ int illm_latent_attn_decode(const float* qa, const void* cache, int dt, const in
                             const int32_t* seq_len, int len_more, float* partial, int nsplit, int B,
                             int H, int R, int dr, float scale, int window, void* stream);
 
+// The same on the matrix cores for a bfloat16 cache with R % 16 == 0, (R + dr) % 8 == 0 and pages of
+// a multiple of 32 rows; cache_t: the transposed copy that illm_latent_rope_store keeps.
+int illm_latent_attn_decode_mfma(const float* qa, const void* cache, const void* cache_t,
+                                 const int32_t* page_table, int table_stride, int page_size,
+                                 int ring, const int32_t* seq_slot, const int32_t* seq_len,
+                                 int len_more, float* partial, int nsplit, int B, int H, int R,
+                                 int dr, float scale, int window, void* stream);
+
 // out[b, h dv + v] = (W_uv[h dv + v, :] . combined sums of (b, h)) * sigmoid(y[b, gate_off + h]).
 int illm_latent_merge_up(const float* partial, int nsplit, const void* wuv, int w_dt, const void* y,
                          int dt, int ncols, int gate_off, void* out, int B, int H, int R, int dv,
                          void* stream);
 
 // ---- routed feed-forward (csrc/moe.hip).  Pair p = t * top + k is token t's k-th choice.
+// z [T, NE] = x [T, K] . w [NE, K]^T for a float32 matrix of few rows (a router's), x of x_dt:
+// float32 products and sums.
+int illm_few_outputs_f32(const void* x, int x_dt, const float* w, float* z, int T, int NE, int K,
+                         void* stream);
+
 // idx, wt [T, top]: the `top` outputs of z [T, NE] (float32) with the largest softmax(z) + corr
 // (corr may be null), in falling order, and their softmax values.  NE <= 512.
 int illm_moe_route(const float* z, const void* corr, int corr_dt, int T, int NE, int top,
                    int32_t* idx, float* wt, void* stream);
 
 // order [NP]: the pairs whose choice is below NEr, grouped by choice; tiles [3 max_tiles + 1]:
-// (expert, first place in order, rows <= illm_moe_tile_rows()) per tile and, last, their number.
-// max_tiles >= min(NP, NP / tile rows + NEr).  NEr <= 512.
+// (expert, first place in order, rows <= tile_rows) per tile and, last, their number.
+// max_tiles >= min(NP, NP / tile_rows + NEr).  NEr <= 512.  illm_moe_tile_rows(): the tile rows
+// that illm_moe_rows takes (illm_moe_rows_mfma: 16, 32 or 64).
 int illm_moe_tile_rows(void);
 int illm_moe_group(const int32_t* idx, int NP, int NEr, int32_t* order, int32_t* tiles,
-                   int max_tiles, void* stream);
+                   int max_tiles, int tile_rows, void* stream);
 
 // Y[p] = X[p / x_div] . W[e_p]^T for every grouped pair p (W [experts][N][K]); gated: W
 // [experts][2 N][K] = [gate | up] rows and Y[p] = silu(X Wg^T) * (X Wu^T).  Y [NP, N] of dt.
 int illm_moe_rows(const void* X, int x_div, const void* W, int dt, int gated, const int32_t* order,
                   const int32_t* tiles, int max_tiles, void* Y, int N, int K, void* stream);
+
+// The same for bfloat16 with K % 32 == 0 and tiles of up to 16, 32 or 64 rows, on the matrix cores.
+int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int gated, int tile_rows,
+                       const int32_t* order, const int32_t* tiles, int max_tiles, void* Y, int N,
+                       int K, void* stream);
 
 // out[t] = sum_k wt[t, k] * (idx[t, k] < NEr ? Y[t top + k] : h[t]) (+ g * shared[t], with
 // g = sigmoid(h[t] . sg), or 1 if sg is null; shared may be null), float32 [T, E].

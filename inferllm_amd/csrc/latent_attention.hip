@@ -24,7 +24,8 @@ latent_rope_store_kernel(void* __restrict__ y, int dt, int ncols, int H, int dn,
                          const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
                          const int32_t* __restrict__ slot_len, void* __restrict__ cache,
                          const int32_t* __restrict__ page_table, int table_stride, int page_size,
-                         int ring, void* __restrict__ c_out, void* __restrict__ kr_out) {
+                         int ring, void* __restrict__ c_out, void* __restrict__ kr_out,
+                         void* __restrict__ cache_t) {
     __shared__ float red[16];
     const int t = blockIdx.x;
     int pos = row_pos[t];
@@ -38,7 +39,7 @@ latent_rope_store_kernel(void* __restrict__ y, int dt, int ncols, int H, int dn,
     ss = block_sum(ss, red);
     const float scale = 1.0f / sqrtf(ss / (float)R + eps);
     bool store = cache != nullptr;
-    size_t dst = 0;
+    size_t dst = 0, dst_t = 0;
     if (store) {
         const int slot = row_slot[t];
         if (ring > 0 && slot_len) {
@@ -51,12 +52,14 @@ latent_rope_store_kernel(void* __restrict__ y, int dt, int ncols, int H, int dn,
             if (ring > 0) lp %= ring;
             const int phys = page_table[(size_t)slot * table_stride + lp];
             dst = ((size_t)phys * page_size + (pos % page_size)) * (size_t)(R + dr);
+            dst_t = (size_t)phys * R * page_size + (pos % page_size);
         }
     }
     for (int i = threadIdx.x; i < R; i += blockDim.x) {
         const float v = (ld_f(y, dt, down + i) * scale) * ld_f(nw, nw_dt, i);
         if (c_out) st_f(c_out, dt, (size_t)t * R + i, v);
         if (store) st_f(cache, dt, dst + i, v);
+        if (store && cache_t) st_f(cache_t, dt, dst_t + (size_t)i * page_size, v);   // [page][dim][row]
     }
     if (pos >= max_pos) pos = max_pos - 1;
     const float* cs = cos_sin ? cos_sin + (size_t)pos * rot : nullptr;   // [rot/2][2]
@@ -90,7 +93,8 @@ extern "C" int illm_latent_rope_store(void* y, int dt, int ncols, int T, int H, 
                                       const int32_t* row_pos, const int32_t* row_slot,
                                       const int32_t* slot_len, void* cache,
                                       const int32_t* page_table, int table_stride, int page_size,
-                                      int ring, void* c_out, void* kr_out, void* stream) {
+                                      int ring, void* c_out, void* kr_out, void* cache_t,
+                                      void* stream) {
     if (T < 0 || H <= 0 || dn < 0 || dr < 0 || R <= 0 || !illm_dtype_ok(dt) || !illm_dtype_ok(norm_dt) ||
         ncols < H * (dn + dr) + R + dr)
         return ILLM_ERR_ARG;
@@ -100,7 +104,7 @@ extern "C" int illm_latent_rope_store(void* y, int dt, int ncols, int T, int H, 
     hipLaunchKernelGGL(latent_rope_store_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, y, dt,
                        ncols, H, dn, dr, R, rot, cos_sin, max_pos, norm_w, norm_dt, eps, row_pos,
                        row_slot, slot_len, cache, page_table, table_stride, page_size, ring, c_out,
-                       kr_out);
+                       kr_out, cache_t);
     return illm_launch_status();
 }
 
@@ -178,10 +182,56 @@ latent_absorb_q_kernel(const void* __restrict__ y, int dt, int ncols, const void
     float* dst = qa + ((size_t)b * H + h) * (size_t)(R + dr);
     for (int r = threadIdx.x; r < R; r += blockDim.x) {
         float acc = 0.f;
+#pragma unroll 8
         for (int d = 0; d < dn; ++d) acc += qs[d] * ld_f(wuk, w_dt, ((size_t)h * dn + d) * R + r);
         dst[r] = acc;
     }
     for (int e = threadIdx.x; e < dr; e += blockDim.x) dst[R + e] = qs[dn + e];
+}
+
+// The same for bfloat16 W_uk with R % 8 == 0 and R <= 512: a thread holds 8 neighbouring latent
+// dims (one 16-byte load a row of W_uk) and takes every (256 / (R / 8))-th plain dim; the groups'
+// sums are added through LDS in group order.
+__global__ void __launch_bounds__(256)
+latent_absorb_q_bf16_kernel(const void* __restrict__ y, int dt, int ncols,
+                            const bf16_t* __restrict__ wuk, float* __restrict__ qa, int H, int dn,
+                            int dr, int R) {
+    extern __shared__ float sm[];
+    float* qs = sm;                       // [dn + dr]
+    float* part = sm + dn + dr;           // [groups][R]
+    const int b = blockIdx.x, h = blockIdx.y;
+    const size_t src = (size_t)b * ncols + (size_t)h * (dn + dr);
+    for (int d = threadIdx.x; d < dn + dr; d += 256) qs[d] = ld_f(y, dt, src + d);
+    __syncthreads();
+    const int per_row = R / 8, groups = 256 / per_row;
+    const int c = threadIdx.x % per_row, g = threadIdx.x / per_row;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+    if (g < groups) {
+        const bf16_t* wp = wuk + (size_t)h * dn * R + c * 8;
+#pragma unroll 4
+        for (int d = g; d < dn; d += groups) {
+            const uint4 u = *(const uint4*)(wp + (size_t)d * R);
+            const float q = qs[d];
+            const uint32_t uw[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[2 * i] += q * __uint_as_float(uw[i] << 16);
+                acc[2 * i + 1] += q * __uint_as_float(uw[i] & 0xffff0000u);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) part[(size_t)g * R + c * 8 + i] = acc[i];
+    }
+    __syncthreads();
+    float* dst = qa + ((size_t)b * H + h) * (size_t)(R + dr);
+    for (int r = threadIdx.x; r < R; r += 256) {
+        float a = 0.f;
+        for (int gg = 0; gg < groups; ++gg) a += part[(size_t)gg * R + r];
+        dst[r] = a;
+    }
+    for (int e = threadIdx.x; e < dr; e += 256) dst[R + e] = qs[dn + e];
 }
 
 extern "C" int illm_latent_absorb_q(const void* y, int dt, int ncols, const void* wuk, int w_dt,
@@ -190,6 +240,15 @@ extern "C" int illm_latent_absorb_q(const void* y, int dt, int ncols, const void
         !illm_dtype_ok(w_dt) || ncols < H * (dn + dr))
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
+    if (w_dt == ILLM_BF16 && R % 8 == 0 && R <= 512 && R >= 8) {
+        const int groups = 256 / (R / 8);
+        const size_t smem = ((size_t)(dn + dr) + (size_t)groups * R) * sizeof(float);
+        if (smem <= 48 * 1024) {
+            hipLaunchKernelGGL(latent_absorb_q_bf16_kernel, dim3(B, H), dim3(256), smem,
+                               (hipStream_t)stream, y, dt, ncols, (const bf16_t*)wuk, qa, H, dn, dr, R);
+            return illm_launch_status();
+        }
+    }
     hipLaunchKernelGGL(latent_absorb_q_kernel, dim3(B, H), dim3(256), (size_t)(dn + dr) * sizeof(float),
                        (hipStream_t)stream, y, dt, ncols, wuk, w_dt, qa, H, dn, dr, R);
     return illm_launch_status();
@@ -394,34 +453,217 @@ extern "C" int illm_latent_attn_decode(const float* qa, const void* cache, int d
 #undef CALL
 }
 
+// The same walk on the matrix cores for a bfloat16 cache (R % 16 == 0, (R + dr) % 8 == 0, pages of
+// a multiple of 32 rows), with a second copy of the latent rows laid out [page][dim][row]
+// (`cache_t`).  A block is one wave: a group of 16 heads, one range of keys, 32 keys at a time.
+// Scores: MFMA 16x16x32 with 16 keys as the A operand (8 neighbouring dims of a cache row, read in
+// operand order straight from memory) and the 16 heads' queries as the B operand (bfloat16, in
+// LDS): lane (r, q) = (lane % 16, lane / 16) is left with head r's scores of keys 4 q .. 4 q + 3 of
+// either half of the 32.  Those 8 weights are the B operand of the second product as they stand:
+// its contraction takes the keys in that order, and the A operand, 16 latent dims by these 8 keys,
+// is two 8-byte loads from the transposed copy.  Keys that are not seen get weight 0 and their
+// loaded values are masked (a freed page may hold anything).  The sums stay in registers
+// (R / 16 accumulators of 4); statistics in float32.
+typedef __bf16 la_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float la_f32x4_t __attribute__((ext_vector_type(4)));
+
+template <int RT>
+__global__ void __launch_bounds__(64)
+latent_decode_mfma_kernel(const float* __restrict__ qa, const bf16_t* __restrict__ cache,
+                          const bf16_t* __restrict__ cache_t,
+                          const int32_t* __restrict__ page_table, int table_stride, int page_size,
+                          int ring, const int32_t* __restrict__ seq_slot,
+                          const int32_t* __restrict__ seq_len, int len_more,
+                          float* __restrict__ partial, int nsplit, int H, int R, int dr, float scale,
+                          int window) {
+    extern __shared__ uint4 qs_raw[];
+    bf16_t* qs = (bf16_t*)qs_raw;                      // [16][D + 8]
+    const int D = R + dr, QS = D + 8;
+    const int b = blockIdx.x, split = blockIdx.y, h0 = blockIdx.z * 16;
+    const int lane = threadIdx.x, r = lane & 15, q = lane >> 4;
+    const int len = seq_len[b] + len_more, slot = seq_slot[b];
+    const int lo = window > 0 ? (len - window > 0 ? len - window : 0) : 0;
+    const int tile0 = lo / 32, tile1 = (len - 1) / 32 + 1;
+    const int per = (tile1 - tile0 + nsplit - 1) / nsplit;
+    const int ta = tile0 + split * per;
+    const int tb = ta + per < tile1 ? ta + per : tile1;
+    for (int e = lane; e < 16 * D; e += 64) {
+        const int hh = e / D, d = e - hh * D;
+        qs[hh * QS + d] = f32_to_bf16(h0 + hh < H ? qa[((size_t)b * H + h0 + hh) * D + d] : 0.f);
+    }
+    __syncthreads();
+    la_f32x4_t o[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) o[rt] = (la_f32x4_t){0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    const la_bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int tile = ta; tile < tb; ++tile) {
+        const int k0 = tile * 32;
+        int lp = k0 / page_size;
+        if (ring > 0) lp %= ring;
+        const int phys = page_table[(size_t)slot * table_stride + lp];
+        const int rowb = k0 % page_size;
+        const bf16_t* kp0 = cache + ((size_t)phys * page_size + rowb + r) * D + 8 * q;
+        const bf16_t* kp1 = kp0 + (size_t)16 * D;
+        la_f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0;
+#pragma unroll 6
+        for (int d0 = 0; d0 < D; d0 += 32) {
+            la_bf16x8_t qv = zero8, ka = zero8, kb = zero8;
+            if (d0 + 8 * q < D) {
+                qv = *(const la_bf16x8_t*)(qs + r * QS + d0 + 8 * q);
+                ka = *(const la_bf16x8_t*)(kp0 + d0);
+                kb = *(const la_bf16x8_t*)(kp1 + d0);
+            }
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qv, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qv, s1, 0, 0, 0);
+        }
+        float sc[8];
+        bool ok[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int p0 = k0 + 4 * q + i, p1 = p0 + 16;
+            ok[i] = p0 >= lo && p0 < len;
+            ok[4 + i] = p1 >= lo && p1 < len;
+            sc[i] = ok[i] ? s0[i] * scale : -INFINITY;
+            sc[4 + i] = ok[4 + i] ? s1[i] * scale : -INFINITY;
+        }
+        float mt = sc[0];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) mt = fmaxf(mt, sc[i]);
+        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float mn = fmaxf(m, mt);
+        const float alpha = m == -INFINITY ? 0.f : expf(m - mn);
+        float pw[8], ls = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            pw[i] = ok[i] ? expf(sc[i] - mn) : 0.f;
+            ls += pw[i];
+        }
+        ls += __shfl_xor(ls, 16, 64);
+        ls += __shfl_xor(ls, 32, 64);
+        l = l * alpha + ls;
+        m = mn;
+        uint4 pu;
+        pu.x = pack_bf16x2(pw[0], pw[1]); pu.y = pack_bf16x2(pw[2], pw[3]);
+        pu.z = pack_bf16x2(pw[4], pw[5]); pu.w = pack_bf16x2(pw[6], pw[7]);
+        const la_bf16x8_t pv = *(const la_bf16x8_t*)&pu;
+        const uint32_t k01 = (ok[0] ? 0xffffu : 0u) | (ok[1] ? 0xffff0000u : 0u);
+        const uint32_t k23 = (ok[2] ? 0xffffu : 0u) | (ok[3] ? 0xffff0000u : 0u);
+        const uint32_t k45 = (ok[4] ? 0xffffu : 0u) | (ok[5] ? 0xffff0000u : 0u);
+        const uint32_t k67 = (ok[6] ? 0xffffu : 0u) | (ok[7] ? 0xffff0000u : 0u);
+        const bf16_t* tp = cache_t + ((size_t)phys * R + r) * page_size + rowb + 4 * q;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            if (rt * 16 < R) {
+                const uint2 c0 = *(const uint2*)(tp + (size_t)rt * 16 * page_size);
+                const uint2 c1 = *(const uint2*)(tp + (size_t)rt * 16 * page_size + 16);
+                uint4 cu;
+                cu.x = c0.x & k01; cu.y = c0.y & k23; cu.z = c1.x & k45; cu.w = c1.y & k67;
+                o[rt][0] *= alpha; o[rt][1] *= alpha; o[rt][2] *= alpha; o[rt][3] *= alpha;
+                o[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const la_bf16x8_t*)&cu, pv, o[rt], 0, 0, 0);
+            }
+        }
+    }
+    // o[rt][i] = sum of head h0 + r over latent dim 16 rt + 4 q + i
+    const int h = h0 + r;
+    if (h < H) {
+        float* dst = partial + (((size_t)b * H + h) * nsplit + split) * (size_t)(R + 2);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            if (rt * 16 < R) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) dst[rt * 16 + 4 * q + i] = o[rt][i];
+            }
+        }
+        if (q == 0) { dst[R] = m; dst[R + 1] = l; }
+    }
+}
+
+extern "C" int illm_latent_attn_decode_mfma(const float* qa, const void* cache, const void* cache_t,
+                                            const int32_t* page_table, int table_stride,
+                                            int page_size, int ring, const int32_t* seq_slot,
+                                            const int32_t* seq_len, int len_more, float* partial,
+                                            int nsplit, int B, int H, int R, int dr, float scale,
+                                            int window, void* stream) {
+    if (B < 0 || H <= 0 || R <= 0 || R > 512 || R % 16 || dr < 0 || (R + dr) % 8 || nsplit < 1 ||
+        nsplit > 65535 || page_size <= 0 || page_size % 32 || table_stride <= 0 || !partial ||
+        !cache || !cache_t)
+        return ILLM_ERR_ARG;
+    if (B == 0) return ILLM_OK;
+    const int groups = (H + 15) / 16;
+    if (groups > 65535) return ILLM_ERR_ARG;
+    const size_t smem = (size_t)16 * (R + dr + 8) * sizeof(bf16_t);
+    const dim3 grid(B, nsplit, groups);
+    hipStream_t st = (hipStream_t)stream;
+#define GO(RT_)                                                                                   \
+    hipLaunchKernelGGL((latent_decode_mfma_kernel<RT_>), grid, dim3(64), smem, st, qa,             \
+                       (const bf16_t*)cache, (const bf16_t*)cache_t, page_table, table_stride,     \
+                       page_size, ring, seq_slot, seq_len, len_more, partial, nsplit, H, R, dr,    \
+                       scale, window)
+    if (R <= 64) GO(4);
+    else if (R <= 128) GO(8);
+    else if (R <= 256) GO(16);
+    else GO(32);
+#undef GO
+    return illm_launch_status();
+}
+
 // grid (B, H): combine the splits, multiply the combined latent sum by W_uv's rows of the head
 // (a wave a value dim, lanes over the latent dims) and by the head's output gate.
 __global__ void __launch_bounds__(256)
 latent_merge_up_kernel(const float* __restrict__ partial, int nsplit, const void* __restrict__ wuv,
                        int w_dt, const void* __restrict__ y, int dt, int ncols, int gate_off,
                        void* __restrict__ out, int H, int R, int dv) {
-    extern __shared__ float ol[];
+    extern __shared__ float ol[];                      // [R] combined sums, then [nsplit] weights
+    float* ws = ol + R;
     const int b = blockIdx.x, h = blockIdx.y;
     const float* base = partial + ((size_t)b * H + h) * nsplit * (size_t)(R + 2);
-    float M = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, base[(size_t)s * (R + 2) + R]);
-    float tot = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-        const float ms = base[(size_t)s * (R + 2) + R];
-        if (ms != -INFINITY) tot += base[(size_t)s * (R + 2) + R + 1] * expf(ms - M);
+    const int w = wave_index(), lane = threadIdx.x & 63;
+    if (w == 0) {
+        // the ranges' (max, weight): lane s holds range s, s + 64, ...; weights exp(m_s - M) / total
+        float M = -INFINITY;
+        for (int s = lane; s < nsplit; s += 64) M = fmaxf(M, base[(size_t)s * (R + 2) + R]);
+        M = wave_max(M);
+        float tot = 0.f;
+        for (int s = lane; s < nsplit; s += 64) {
+            const float ms = base[(size_t)s * (R + 2) + R];
+            const float e = ms == -INFINITY ? 0.f : expf(ms - M);
+            ws[s] = e;
+            tot += base[(size_t)s * (R + 2) + R + 1] * e;
+        }
+        tot = wave_sum(tot);
+        for (int s = lane; s < nsplit; s += 64) ws[s] = ws[s] / tot;
     }
+    __syncthreads();
     for (int r = threadIdx.x; r < R; r += 256) {
         float a = 0.f;
-        for (int s = 0; s < nsplit; ++s) {
-            const float ms = base[(size_t)s * (R + 2) + R];
-            if (ms != -INFINITY) a += base[(size_t)s * (R + 2) + r] * expf(ms - M);
-        }
-        ol[r] = a / tot;
+        for (int s = 0; s < nsplit; ++s) a += base[(size_t)s * (R + 2) + r] * ws[s];
+        ol[r] = a;
     }
     __syncthreads();
     const float g = ld_f(y, dt, (size_t)b * ncols + gate_off + h);
     const float gate = 1.0f / (1.0f + expf(-g));
-    const int w = wave_index(), lane = threadIdx.x & 63;
+    if (w_dt == ILLM_BF16 && R % 8 == 0) {
+        // 16-byte loads: a lane takes 8 neighbouring latent dims of a row of W_uv
+        const bf16_t* wp = (const bf16_t*)wuv;
+        for (int v = w; v < dv; v += 4) {
+            const size_t wr = ((size_t)h * dv + v) * R;
+            float dot = 0.f;
+            for (int r = lane * 8; r < R; r += 512) {
+                const uint4 u = *(const uint4*)(wp + wr + r);
+                const uint32_t uw[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    dot += __uint_as_float(uw[i] << 16) * ol[r + 2 * i];
+                    dot += __uint_as_float(uw[i] & 0xffff0000u) * ol[r + 2 * i + 1];
+                }
+            }
+            dot = wave_sum(dot);
+            if (lane == 0) st_f(out, dt, (size_t)b * H * dv + (size_t)h * dv + v, dot * gate);
+        }
+        return;
+    }
     for (int v = w; v < dv; v += 4) {
         const size_t wr = ((size_t)h * dv + v) * R;
         float dot = 0.f;
@@ -438,7 +680,7 @@ extern "C" int illm_latent_merge_up(const float* partial, int nsplit, const void
         !illm_dtype_ok(w_dt) || gate_off < 0 || gate_off + H > ncols)
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
-    hipLaunchKernelGGL(latent_merge_up_kernel, dim3(B, H), dim3(256), (size_t)R * sizeof(float),
+    hipLaunchKernelGGL(latent_merge_up_kernel, dim3(B, H), dim3(256), (size_t)(R + nsplit) * sizeof(float),
                        (hipStream_t)stream, partial, nsplit, wuv, w_dt, y, dt, ncols, gate_off, out,
                        H, R, dv);
     return illm_launch_status();

@@ -13,6 +13,31 @@
 #define MOE_TILE 8
 
 // ---------------------------------------------------------------- router
+// z[t, e] = sum_k x[t, k] w[e, k] with a float32 matrix of few rows (a router): a wave an output,
+// lanes over K, float32 products and sums in an order fixed by K.  grid (T, ceil(NE / 4)).
+__global__ void __launch_bounds__(256)
+few_outputs_f32_kernel(const void* __restrict__ x, int x_dt, const float* __restrict__ w,
+                       float* __restrict__ z, int NE, int K) {
+    const size_t t = blockIdx.x;
+    const int e = blockIdx.y * 4 + wave_index(), lane = threadIdx.x & 63;
+    if (e >= NE) return;
+    const float* wr = w + (size_t)e * K;
+    float acc = 0.f;
+#pragma unroll 4
+    for (int k = lane; k < K; k += 64) acc += ld_f(x, x_dt, t * K + k) * wr[k];
+    acc = wave_sum(acc);
+    if (lane == 0) z[t * NE + e] = acc;
+}
+
+extern "C" int illm_few_outputs_f32(const void* x, int x_dt, const float* w, float* z, int T, int NE,
+                                    int K, void* stream) {
+    if (T < 0 || NE <= 0 || NE > 65535 * 4 || K <= 0 || !illm_dtype_ok(x_dt)) return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    hipLaunchKernelGGL(few_outputs_f32_kernel, dim3(T, (NE + 3) / 4), dim3(256), 0, (hipStream_t)stream,
+                       x, x_dt, w, z, NE, K);
+    return illm_launch_status();
+}
+
 // One wave per token: s = softmax(z) over all NE outputs (float32), choice score = s + correction,
 // the `top` largest choice scores (lowest index on ties) in falling order; weights are s.
 #define MOE_EPL 8                                   // outputs a lane holds: up to 512 experts
@@ -82,7 +107,7 @@ extern "C" int illm_moe_route(const float* z, const void* corr, int corr_dt, int
 #define MOE_MAX_EXPERTS 512
 __global__ void __launch_bounds__(1024)
 moe_group_kernel(const int32_t* __restrict__ idx, int NP, int NEr, int32_t* __restrict__ order,
-                 int32_t* __restrict__ tiles, int max_tiles) {
+                 int32_t* __restrict__ tiles, int max_tiles, int tile_rows) {
     __shared__ int cnt[MOE_MAX_EXPERTS], offs[MOE_MAX_EXPERTS], tile0[MOE_MAX_EXPERTS + 1];
     for (int e = threadIdx.x; e < NEr; e += blockDim.x) cnt[e] = 0;
     __syncthreads();
@@ -96,7 +121,7 @@ moe_group_kernel(const int32_t* __restrict__ idx, int NP, int NEr, int32_t* __re
         for (int e = 0; e < NEr; ++e) {
             offs[e] = o; tile0[e] = tl;
             o += cnt[e];
-            tl += (cnt[e] + MOE_TILE - 1) / MOE_TILE;
+            tl += (cnt[e] + tile_rows - 1) / tile_rows;
         }
         tile0[NEr] = tl;
         tiles[3 * (size_t)max_tiles] = tl < max_tiles ? tl : max_tiles;
@@ -104,10 +129,10 @@ moe_group_kernel(const int32_t* __restrict__ idx, int NP, int NEr, int32_t* __re
     __syncthreads();
     for (int e = threadIdx.x; e < NEr; e += blockDim.x) {
         const int n = cnt[e];
-        for (int s = 0, i = tile0[e]; s < n && i < max_tiles; s += MOE_TILE, ++i) {
+        for (int s = 0, i = tile0[e]; s < n && i < max_tiles; s += tile_rows, ++i) {
             tiles[3 * (size_t)i] = e;
             tiles[3 * (size_t)i + 1] = offs[e] + s;
-            tiles[3 * (size_t)i + 2] = n - s < MOE_TILE ? n - s : MOE_TILE;
+            tiles[3 * (size_t)i + 2] = n - s < tile_rows ? n - s : tile_rows;
         }
     }
     __syncthreads();
@@ -122,40 +147,38 @@ moe_group_kernel(const int32_t* __restrict__ idx, int NP, int NEr, int32_t* __re
 extern "C" int illm_moe_tile_rows(void) { return MOE_TILE; }
 
 extern "C" int illm_moe_group(const int32_t* idx, int NP, int NEr, int32_t* order, int32_t* tiles,
-                              int max_tiles, void* stream) {
-    if (NP < 0 || NEr < 0 || NEr > MOE_MAX_EXPERTS || max_tiles < 0) return ILLM_ERR_ARG;
+                              int max_tiles, int tile_rows, void* stream) {
+    if (NP < 0 || NEr < 0 || NEr > MOE_MAX_EXPERTS || max_tiles < 0 || tile_rows <= 0)
+        return ILLM_ERR_ARG;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, idx, NP, NEr,
-                       order, tiles, max_tiles);
+                       order, tiles, max_tiles, tile_rows);
     return illm_launch_status();
 }
 
 // ---------------------------------------------------------------- the experts' products
-// Four elements of a row as float32; V = 4: one 8- or 16-byte load, V = 1: element by element.
-template <int DT>
-__device__ __forceinline__ float4 ld4(const void* p, size_t i) {
-    if (DT == ILLM_BF16) {
-        const uint2 u = *(const uint2*)((const bf16_t*)p + i);
-        return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
-                           __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
-    }
-    return *(const float4*)((const float*)p + i);
-}
-
-template <int DT>
-__device__ __forceinline__ float ld1(const void* p, size_t i) {
-    return DT == ILLM_BF16 ? bf16_to_f32(((const bf16_t*)p)[i]) : ((const float*)p)[i];
-}
-
-// Sum over the wave of n <= MOE_TILE values per lane.
-__device__ __forceinline__ void wave_sums(float* v, int n) {
+// V elements of a row as float32: bfloat16 V = 8 (one 16-byte load), float32 V = 4, or V = 1.
+template <int DT, int V>
+__device__ __forceinline__ void ldv(const void* p, size_t i, float* o) {
+    if (V == 8) {
+        const uint4 u = *(const uint4*)((const bf16_t*)p + i);
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
-    for (int r = 0; r < MOE_TILE; ++r)
-        if (r < n) v[r] = wave_sum(v[r]);
+        for (int j = 0; j < 4; ++j) {
+            o[2 * j] = __uint_as_float(w[j] << 16);
+            o[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        }
+    } else if (V == 4) {
+        const float4 f = *(const float4*)((const float*)p + i);
+        o[0] = f.x; o[1] = f.y; o[2] = f.z; o[3] = f.w;
+    } else {
+        o[0] = DT == ILLM_BF16 ? bf16_to_f32(((const bf16_t*)p)[i]) : ((const float*)p)[i];
+    }
 }
 
 // grid (tiles, column groups).  X rows: pair p reads row p / x_div of X (x_div = top for the
 // tokens' rows, 1 for rows that are per pair already).  GATED: W holds [gate (N) | up (N)] rows per
-// expert and Y = silu(X Wg^T) * (X Wu^T); else Y = X W^T.  Y rows are per pair.
+// expert and Y = silu(X Wg^T) * (X Wu^T); else Y = X W^T.  Y rows are per pair.  A wave takes two
+// columns at a time, so that their rows of W are in flight together.
 template <int DT, int V, bool GATED>
 __global__ void __launch_bounds__(256)
 moe_rows_kernel(const void* __restrict__ X, int x_div, const void* __restrict__ W,
@@ -171,55 +194,54 @@ moe_rows_kernel(const void* __restrict__ X, int x_div, const void* __restrict__ 
     for (int r = 0; r < MOE_TILE; ++r) pair[r] = r < n ? order[first + r] : 0;
     const size_t wrows = GATED ? 2 * (size_t)N : (size_t)N;
     const int c_end = min(N, (int)(blockIdx.y + 1) * cols_per_block);
-    for (int col = blockIdx.y * cols_per_block + w; col < c_end; col += 4) {
-        const size_t wa = ((size_t)e * wrows + col) * K, wb = wa + (size_t)N * K;
-        float a[MOE_TILE], g[MOE_TILE];
+    for (int col = blockIdx.y * cols_per_block + 2 * w; col < c_end; col += 8) {
+        const bool two = col + 1 < c_end;
+        const size_t wa0 = ((size_t)e * wrows + col) * K, wa1 = two ? wa0 + K : wa0;
+        const size_t up = (size_t)N * K;
+        float a[2][MOE_TILE], g[2][MOE_TILE];
 #pragma unroll
-        for (int r = 0; r < MOE_TILE; ++r) { a[r] = 0.f; g[r] = 0.f; }
+        for (int r = 0; r < MOE_TILE; ++r) { a[0][r] = a[1][r] = 0.f; g[0][r] = g[1][r] = 0.f; }
+#pragma unroll 2
         for (int k = lane * V; k < K; k += 64 * V) {
-            if (V == 4) {
-                const float4 w0 = ld4<DT>(W, wa + k);
-                float4 w1 = w0;
-                if (GATED) w1 = ld4<DT>(W, wb + k);
+            float w0[V], w1[V], u0[V], u1[V];
+            ldv<DT, V>(W, wa0 + k, w0);
+            ldv<DT, V>(W, wa1 + k, w1);
+            if (GATED) { ldv<DT, V>(W, wa0 + up + k, u0); ldv<DT, V>(W, wa1 + up + k, u1); }
 #pragma unroll
-                for (int r = 0; r < MOE_TILE; ++r) {
-                    if (r < n) {
-                        const float4 x = ld4<DT>(X, (size_t)(pair[r] / x_div) * K + k);
-                        a[r] += x.x * w0.x; a[r] += x.y * w0.y; a[r] += x.z * w0.z; a[r] += x.w * w0.w;
-                        if (GATED) {
-                            g[r] += x.x * w1.x; g[r] += x.y * w1.y; g[r] += x.z * w1.z; g[r] += x.w * w1.w;
-                        }
-                    }
-                }
-            } else {
-                const float w0 = ld1<DT>(W, wa + k);
-                const float w1 = GATED ? ld1<DT>(W, wb + k) : 0.f;
+            for (int r = 0; r < MOE_TILE; ++r) {
+                if (r < n) {
+                    float x[V];
+                    ldv<DT, V>(X, (size_t)(pair[r] / x_div) * K + k, x);
 #pragma unroll
-                for (int r = 0; r < MOE_TILE; ++r) {
-                    if (r < n) {
-                        const float x = ld1<DT>(X, (size_t)(pair[r] / x_div) * K + k);
-                        a[r] += x * w0;
-                        if (GATED) g[r] += x * w1;
+                    for (int j = 0; j < V; ++j) {
+                        a[0][r] += x[j] * w0[j];
+                        a[1][r] += x[j] * w1[j];
+                        if (GATED) { g[0][r] += x[j] * u0[j]; g[1][r] += x[j] * u1[j]; }
                     }
                 }
             }
         }
-        wave_sums(a, n);
-        if (GATED) wave_sums(g, n);
-        if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < MOE_TILE; ++r) {
+            if (r < n) {
+                a[0][r] = wave_sum(a[0][r]); a[1][r] = wave_sum(a[1][r]);
+                if (GATED) { g[0][r] = wave_sum(g[0][r]); g[1][r] = wave_sum(g[1][r]); }
+            }
+        }
+        if (lane < 2 && (lane == 0 || two)) {
 #pragma unroll
             for (int r = 0; r < MOE_TILE; ++r) {
                 if (r < n) {
-                    float v = a[r];
+                    float v = lane ? a[1][r] : a[0][r];
                     if (GATED) {
                         // the products take the activations' type before the activation, as a
                         // product of its own would leave them
-                        float gate = a[r], up = g[r];
-                        if (DT == ILLM_BF16) { gate = bf16_to_f32(f32_to_bf16(gate)); up = bf16_to_f32(f32_to_bf16(up)); }
-                        v = (gate / (1.0f + expf(-gate))) * up;
+                        float gate = v, upv = lane ? g[1][r] : g[0][r];
+                        if (DT == ILLM_BF16) { gate = bf16_to_f32(f32_to_bf16(gate)); upv = bf16_to_f32(f32_to_bf16(upv)); }
+                        v = (gate / (1.0f + expf(-gate))) * upv;
                     }
-                    if (DT == ILLM_BF16) ((bf16_t*)Y)[(size_t)pair[r] * N + col] = f32_to_bf16(v);
-                    else ((float*)Y)[(size_t)pair[r] * N + col] = v;
+                    if (DT == ILLM_BF16) ((bf16_t*)Y)[(size_t)pair[r] * N + col + lane] = f32_to_bf16(v);
+                    else ((float*)Y)[(size_t)pair[r] * N + col + lane] = v;
                 }
             }
         }
@@ -237,17 +259,125 @@ extern "C" int illm_moe_rows(const void* X, int x_div, const void* W, int dt, in
     const dim3 grid(max_tiles, (N + cols - 1) / cols);
     if (grid.y > 65535) return ILLM_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    const bool vec = K % 4 == 0;
 #define GO(DT_, V_, G_)                                                                          \
     hipLaunchKernelGGL((moe_rows_kernel<DT_, V_, G_>), grid, dim3(256), 0, st, X, x_div, W, order, \
                        tiles, max_tiles, Y, N, K, cols)
     if (dt == ILLM_BF16) {
-        if (vec) { if (gated) GO(ILLM_BF16, 4, true); else GO(ILLM_BF16, 4, false); }
+        if (K % 8 == 0) { if (gated) GO(ILLM_BF16, 8, true); else GO(ILLM_BF16, 8, false); }
         else { if (gated) GO(ILLM_BF16, 1, true); else GO(ILLM_BF16, 1, false); }
     } else {
-        if (vec) { if (gated) GO(ILLM_F32, 4, true); else GO(ILLM_F32, 4, false); }
+        if (K % 4 == 0) { if (gated) GO(ILLM_F32, 4, true); else GO(ILLM_F32, 4, false); }
         else { if (gated) GO(ILLM_F32, 1, true); else GO(ILLM_F32, 1, false); }
     }
+#undef GO
+    return illm_launch_status();
+}
+
+// The same products for tiles of up to 16 MT pairs on the matrix cores (bfloat16, K % 32 == 0):
+// MFMA 16x16x32 with 16 rows of W as the A operand and 16 of the tile's X rows as the B operand,
+// both read in operand order straight from memory (lane (r, q) = (lane % 16, lane / 16) holds 8
+// consecutive k of row r at k0 + 8 q; the tile's X rows stay in the caches, W is read once a
+// tile).  A wave takes NT groups of 16 output columns at a time and all MT row groups, so an X
+// operand serves NT (gated: 2 NT) products; the sum over K runs in one fixed order, so a row's
+// result does not depend on its tile.  grid (tiles, column groups of 64 NT).
+typedef __bf16 moe_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float moe_f32x4_t __attribute__((ext_vector_type(4)));
+
+template <int MT, int NT, bool GATED>
+__global__ void __launch_bounds__(256)
+moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __restrict__ W,
+                     const int32_t* __restrict__ order, const int32_t* __restrict__ tiles,
+                     int max_tiles, bf16_t* __restrict__ Y, int N, int K) {
+    const int tile = blockIdx.x;
+    if (tile >= tiles[3 * (size_t)max_tiles]) return;
+    const int e = tiles[3 * (size_t)tile], first = tiles[3 * (size_t)tile + 1];
+    const int n = tiles[3 * (size_t)tile + 2];
+    const int w = wave_index(), lane = threadIdx.x & 63;
+    const int r = lane & 15, q = lane >> 4;
+    int pair[MT];
+    const bf16_t* xp[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int i = mt * 16 + r;
+        pair[mt] = order[first + (i < n ? i : n - 1)];          // rows beyond the tile: read, not written
+        xp[mt] = X + (size_t)(pair[mt] / x_div) * K + q * 8;
+    }
+    const size_t wrows = GATED ? 2 * (size_t)N : (size_t)N;
+    const int n0 = (blockIdx.y * 4 + w) * 16 * NT;
+    if (n0 >= N) return;
+    const bf16_t* wa[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int wr = n0 + nt * 16 + r < N ? n0 + nt * 16 + r : N - 1;
+        wa[nt] = W + ((size_t)e * wrows + wr) * K + q * 8;
+    }
+    const size_t up = (size_t)N * K;
+    moe_f32x4_t a[NT][MT], g[NT][MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            a[nt][mt] = (moe_f32x4_t){0.f, 0.f, 0.f, 0.f};
+            g[nt][mt] = a[nt][mt];
+        }
+    for (int k = 0; k < K; k += 32) {
+        moe_bf16x8_t w0[NT], w1[NT], x[MT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            w0[nt] = *(const moe_bf16x8_t*)(wa[nt] + k);
+            if (GATED) w1[nt] = *(const moe_bf16x8_t*)(wa[nt] + up + k);
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) x[mt] = *(const moe_bf16x8_t*)(xp[mt] + k);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                a[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[nt], x[mt], a[nt][mt], 0, 0, 0);
+                if (GATED)
+                    g[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[nt], x[mt], g[nt][mt], 0, 0, 0);
+            }
+    }
+    // a[nt][mt][i] belongs to the pair of row mt * 16 + r and column n0 + 16 nt + 4 q + i
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        if (mt * 16 + r >= n) continue;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int col = n0 + 16 * nt + 4 * q + i;
+                if (col >= N) continue;
+                float v = a[nt][mt][i];
+                if (GATED) {
+                    const float gate = bf16_to_f32(f32_to_bf16(a[nt][mt][i]));
+                    const float upv = bf16_to_f32(f32_to_bf16(g[nt][mt][i]));
+                    v = (gate / (1.0f + expf(-gate))) * upv;
+                }
+                Y[(size_t)pair[mt] * N + col] = f32_to_bf16(v);
+            }
+    }
+}
+
+extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int gated, int tile_rows,
+                                  const int32_t* order, const int32_t* tiles, int max_tiles,
+                                  void* Y, int N, int K, void* stream) {
+    if (x_div <= 0 || N <= 0 || K <= 0 || K % 32 || max_tiles < 0 || max_tiles > 2147483647 / 3 ||
+        (tile_rows != 16 && tile_rows != 32 && tile_rows != 64))
+        return ILLM_ERR_ARG;
+    if (max_tiles == 0) return ILLM_OK;
+    hipStream_t st = (hipStream_t)stream;
+#define GO(MT_, NT_, G_)                                                                           \
+    do {                                                                                           \
+        const dim3 grid(max_tiles, (N + 64 * NT_ - 1) / (64 * NT_));                               \
+        if (grid.y > 65535) return ILLM_ERR_ARG;                                                   \
+        hipLaunchKernelGGL((moe_rows_mfma_kernel<MT_, NT_, G_>), grid, dim3(256), 0, st,           \
+                           (const bf16_t*)X, x_div, (const bf16_t*)W, order, tiles, max_tiles,     \
+                           (bf16_t*)Y, N, K);                                                      \
+    } while (0)
+    if (tile_rows == 16) { if (gated) GO(1, 4, true); else GO(1, 4, false); }
+    else if (tile_rows == 32) { if (gated) GO(2, 4, true); else GO(2, 4, false); }
+    else { if (gated) GO(4, 2, true); else GO(4, 4, false); }
 #undef GO
     return illm_launch_status();
 }

@@ -1045,12 +1045,17 @@ def latent_rope_store(y: torch.Tensor, H: int, dn: int, dr: int, R: int, rot: in
                       row_pos: torch.Tensor, row_slot: torch.Tensor,
                       slot_len: Optional[torch.Tensor], cache: Optional[torch.Tensor],
                       page_table: Optional[torch.Tensor], page_size: int, ring: int,
-                      want_rows: bool):
+                      want_rows: bool, cache_t: Optional[torch.Tensor] = None):
     """Rows y [T, >= H (dn + dr) + R + dr] = [q | down | ...]: the latent (first R of `down`) is
     RMS-normed, the key part (last dr) and every q head's last dr dims are rotated (pairs
     (2i, 2i+1), i < rot/2) at row_pos, q in place; latent and key part are stored in the paged
-    cache [pages, page_size, R + dr].  `want_rows`: also return them as (c [T, R], kr [T, dr])."""
-    _gpu(y, cos_sin, norm_w, row_pos, row_slot, slot_len, cache, page_table)
+    cache [pages, page_size, R + dr] (and the latent alone a second time, transposed, in
+    cache_t [pages, R, page_size, 1] if given).  `want_rows`: also return them as (c [T, R],
+    kr [T, dr])."""
+    _gpu(y, cos_sin, norm_w, row_pos, row_slot, slot_len, cache, page_table, cache_t)
+    _need(cache_t is None or (cache is not None and cache_t.dtype == y.dtype and
+                              cache_t.shape == (cache.shape[0], R, page_size, 1)),
+          "latent_rope_store: the transposed copy must be [pages, R, page_size, 1]")
     T, ncols = y.shape
     _i32(row_pos, T); _i32(row_slot, T); _i32(slot_len); _i32(page_table)
     _need(ncols >= H * (dn + dr) + R + dr, "latent_rope_store: rows too short")
@@ -1072,7 +1077,8 @@ def latent_rope_store(y: torch.Tensor, H: int, dn: int, dr: int, R: int, rot: in
     _check(_lib().illm_latent_rope_store(
         _p(y), _code(y), ncols, T, H, dn, dr, R, rot, _p(cos_sin), max_pos, _p(norm_w),
         _code(norm_w), ctypes.c_float(eps), _p(row_pos), _p(row_slot), _p(slot_len), _p(cache),
-        _p(page_table), stride, page_size, ring, _p(c), _p(kr), _stream()), "latent_rope_store")
+        _p(page_table), stride, page_size, ring, _p(c), _p(kr), _p(cache_t), _stream()),
+        "latent_rope_store")
     return c, kr
 
 
@@ -1101,17 +1107,27 @@ def latent_gate(attn: torch.Tensor, y: torch.Tensor, gate_off: int, H: int, dv: 
     return out
 
 
-def latent_decode_splits(B: int, H: int, longest: int) -> int:
+def latent_decode_splits(B: int, H: int, longest: int, mfma: bool = False) -> int:
     """Ranges the keys of a one-token step are cut into: about as many blocks as the chip has
-    compute units, at most 16 ranges, none shorter than 64 keys."""
+    compute units, at most 16 ranges, none shorter than 64 keys; for the matrix-core kernel, whose
+    blocks are single waves, about four waves a compute unit, at most 64 ranges of 32 keys or more."""
+    if mfma:
+        return max(1, min(-(-1024 // max(1, B * -(-H // 16))), 64, (longest + 31) // 32))
     groups = -(-H // (16 if H >= 16 else 8 if H >= 8 else 4))
     return max(1, min(-(-256 // max(1, B * groups)), 16, (longest + 63) // 64))
+
+
+def latent_decode_mfma_fits(cache: torch.Tensor, cache_t: Optional[torch.Tensor], R: int, dr: int,
+                            page_size: int) -> bool:
+    return (cache_t is not None and cache.dtype == torch.bfloat16 and R % 16 == 0 and R <= 512
+            and (R + dr) % 8 == 0 and page_size % 32 == 0)
 
 
 def latent_attn_decode(y: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor, gate_off: int,
                        cache: torch.Tensor, page_table: torch.Tensor, page_size: int, ring: int,
                        seq_slot: torch.Tensor, seq_len: torch.Tensor, len_more: int, H: int, dn: int,
-                       dr: int, R: int, dv: int, scale: float, window: int, nsplit: int) -> torch.Tensor:
+                       dr: int, R: int, dv: int, scale: float, window: int, nsplit: int,
+                       cache_t: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One token per sequence over the latent cache, never building a head's keys or values:
     queries are taken through W_uk first, the weighted sums of latent rows through W_uv after,
     then the head's output gate.  y [B, ...] = [q (rotated) | down | gate]; token b sees
@@ -1126,10 +1142,19 @@ def latent_attn_decode(y: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor, 
     _check(_lib().illm_latent_absorb_q(_p(y), _code(y), y.shape[1], _p(w_uk), _code(w_uk), _p(qa),
                                        B, H, dn, dr, R, _stream()), "latent_absorb_q")
     partial = torch.empty((B, H, nsplit, R + 2), dtype=torch.float32, device=y.device)
-    _check(_lib().illm_latent_attn_decode(
+    if cache_t is not None:
+        _need(latent_decode_mfma_fits(cache, cache_t, R, dr, page_size) and
+              cache_t.shape == (cache.shape[0], R, page_size, 1) and cache_t.is_contiguous(),
+              "latent_attn_decode: the transposed copy is not taken")
+        _check(_lib().illm_latent_attn_decode_mfma(
+            _p(qa), _p(cache), _p(cache_t), _p(page_table), page_table.shape[1], page_size, ring,
+            _p(seq_slot), _p(seq_len), len_more, _p(partial), nsplit, B, H, R, dr,
+            ctypes.c_float(scale), window, _stream()), f"latent_attn_decode_mfma (latent {R}+{dr})")
+    else:
+        _check(_lib().illm_latent_attn_decode(
         _p(qa), _p(cache), _code(cache), _p(page_table), page_table.shape[1], page_size, ring,
-        _p(seq_slot), _p(seq_len), len_more, _p(partial), nsplit, B, H, R, dr, ctypes.c_float(scale),
-        window, _stream()), f"latent_attn_decode (latent {R}+{dr})")
+            _p(seq_slot), _p(seq_len), len_more, _p(partial), nsplit, B, H, R, dr, ctypes.c_float(scale),
+            window, _stream()), f"latent_attn_decode (latent {R}+{dr})")
     out = torch.empty((B, H * dv), dtype=y.dtype, device=y.device)
     _check(_lib().illm_latent_merge_up(_p(partial), nsplit, _p(w_uv), _code(w_uv), _p(y), _code(y),
                                        y.shape[1], gate_off, _p(out), B, H, R, dv, _stream()),
@@ -1138,6 +1163,19 @@ def latent_attn_decode(y: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor, 
 
 
 # ------------------------------------------------------------------ routed feed-forward
+def few_outputs_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """float32 x . w^T for a float32 matrix w [outputs, K] of few rows (a router's) and rows x of
+    either type; products and sums in float32."""
+    _gpu(x, w)
+    _need(w.dtype == torch.float32 and x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1],
+          f"few_outputs_f32: x {tuple(x.shape)} against float32 w {tuple(w.shape)}")
+    T, K = x.shape
+    z = torch.empty((T, w.shape[0]), dtype=torch.float32, device=x.device)
+    _check(_lib().illm_few_outputs_f32(_p(x), _code(x), _p(w), _p(z), T, w.shape[0], K, _stream()),
+           "few_outputs_f32")
+    return z
+
+
 def moe_route(z: torch.Tensor, correction: Optional[torch.Tensor], top: int):
     """(idx int32 [T, top], weight float32 [T, top]): per row of the router's float32 outputs z
     the `top` largest softmax(z) + correction, and their softmax values."""
@@ -1153,6 +1191,10 @@ def moe_route(z: torch.Tensor, correction: Optional[torch.Tensor], top: int):
     return idx, wt
 
 
+MOE_MFMA_FROM = 8        # (token, choice) pairs an expert on average from which the experts' products
+                         # run on the matrix cores (below: a wave a column, lanes over K)
+
+
 def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
     """Y [T * top, E]: for every (token, choice) pair whose choice is one of the stacked experts
     (w_gate_up [experts, 2 F, E] = [gate | up], w_down [experts, E, F]) the expert's
@@ -1166,18 +1208,29 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gate_up: torch.Tensor, w_d
           and w_gate_up.dtype == h.dtype and w_down.dtype == h.dtype and idx.shape[0] == T,
           "moe_experts: shapes or dtypes")
     NP = T * top
-    rows = _lib().illm_moe_tile_rows()
+    F = F2 // 2
+    # many pairs an expert (prompts): tiles of up to 64 rows on the matrix cores; few (single
+    # tokens): tiles of 8 rows, a wave a column, which reads an expert's matrices once
+    per_expert = NP / max(1, n_exp)
+    mfma = h.dtype == torch.bfloat16 and E % 32 == 0 and F % 32 == 0 and per_expert >= MOE_MFMA_FROM
+    rows = (64 if per_expert >= 48 else 32 if per_expert >= 24 else 16) if mfma else _lib().illm_moe_tile_rows()
     max_tiles = max(1, min(NP, NP // rows + n_exp))
     order = torch.empty((NP,), dtype=torch.int32, device=h.device)
     tiles = torch.empty((3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
-    _check(_lib().illm_moe_group(_p(idx), NP, n_exp, _p(order), _p(tiles), max_tiles, _stream()),
-           "moe_group")
-    act = torch.empty((NP, F2 // 2), dtype=h.dtype, device=h.device)
-    _check(_lib().illm_moe_rows(_p(h), top, _p(w_gate_up), _code(h), 1, _p(order), _p(tiles),
-                                max_tiles, _p(act), F2 // 2, E, _stream()), "moe_rows (gate|up)")
+    _check(_lib().illm_moe_group(_p(idx), NP, n_exp, _p(order), _p(tiles), max_tiles, rows,
+                                 _stream()), "moe_group")
+    act = torch.empty((NP, F), dtype=h.dtype, device=h.device)
     y = torch.empty((NP, E), dtype=h.dtype, device=h.device)
+    if mfma:
+        _check(_lib().illm_moe_rows_mfma(_p(h), top, _p(w_gate_up), 1, rows, _p(order), _p(tiles),
+                                         max_tiles, _p(act), F, E, _stream()), "moe_rows_mfma (gate|up)")
+        _check(_lib().illm_moe_rows_mfma(_p(act), 1, _p(w_down), 0, rows, _p(order), _p(tiles),
+                                         max_tiles, _p(y), E, F, _stream()), "moe_rows_mfma (down)")
+        return y
+    _check(_lib().illm_moe_rows(_p(h), top, _p(w_gate_up), _code(h), 1, _p(order), _p(tiles),
+                                max_tiles, _p(act), F, E, _stream()), "moe_rows (gate|up)")
     _check(_lib().illm_moe_rows(_p(act), 1, _p(w_down), _code(h), 0, _p(order), _p(tiles),
-                                max_tiles, _p(y), E, F2 // 2, _stream()), "moe_rows (down)")
+                                max_tiles, _p(y), E, F, _stream()), "moe_rows (down)")
     return y
 
 

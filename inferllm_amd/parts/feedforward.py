@@ -171,7 +171,7 @@ class RoutedExperts(FeedForward):
                 self.w_sg = take("shared.sg").reshape(-1).contiguous()
 
     def forward(self, h, ctx: StepContext):
-        z = ops.linear(h, self.w_router, out_dtype=torch.float32)
+        z = ops.few_outputs_f32(h, self.w_router)
         idx, weight = ops.moe_route(z, self.correction, self.top)
         y = ops.moe_experts(h, idx, self.w_gate_up, self.w_down) if self.n_real else None
         shared = None

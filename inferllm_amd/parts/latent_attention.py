@@ -55,6 +55,9 @@ class LatentAttention(Mixer):
         self.q_cols = self.H * (self.dn + self.dr)
         self.gate_off = self.q_cols + self.R + self.dr
         self.w_in = self.w_up = self.w_uk = self.w_uv = self.w_o = self.norm_w = None
+        # set by `load` (which sees the engine's dtype): keep the latent rows a second time,
+        # transposed, for the single-token kernel on the matrix cores
+        self.transposed = False
 
     def shapes(self) -> Dict[str, TensorWant]:
         out = {"q": TensorWant((self.q_cols, self.E)),
@@ -68,8 +71,10 @@ class LatentAttention(Mixer):
         return out
 
     def kv_spec(self) -> KVSpec:
-        return KVSpec("window" if self.window else "full",
-                      (TokenTensor("latent", (self.R + self.dr,)),), self.window)
+        kept = (TokenTensor("latent", (self.R + self.dr,)),)
+        if self.transposed:
+            kept += (TokenTensor("latent_t", (self.R, 1)),)     # stored [page][dim][row][1]
+        return KVSpec("window" if self.window else "full", kept, self.window)
 
     def head_width(self, dtype: torch.dtype) -> int:
         """The common width the heads are padded to for the prompt attention kernels."""
@@ -92,11 +97,15 @@ class LatentAttention(Mixer):
         self.w_up = _fuse([self.w_uk, self.w_uv])
         self.w_o = ops.decode_weight(self._take(tensors, "o").contiguous(), "plain", self.decode_copies)
         self.norm_w = self._take(tensors, "dkv_norm").contiguous()
+        self.transposed = (self.w_uk.dtype == torch.bfloat16 and self.R % 16 == 0
+                           and (self.R + self.dr) % 8 == 0)
 
     def forward(self, h, ctx: StepContext, line, writes_cache, position):
         H, dn, dr, dv, R = self.H, self.dn, self.dr, self.dv, self.R
         kept, group = ctx.cache.token_line(line)
-        cache = kept["latent"]
+        cache, cache_t = kept["latent"], kept.get("latent_t")
+        if cache_t is not None and not ops.latent_decode_mfma_fits(cache, cache_t, R, dr, group.page_size):
+            cache_t = None
         window = self.window or 0
         table = position.table(ctx.device) if position is not None else None
         rot = position.rotary_dim if position is not None else 0
@@ -107,7 +116,8 @@ class LatentAttention(Mixer):
         c, kr = ops.latent_rope_store(
             y, H, dn, dr, R, rot, table, self.norm_w, self.eps, ctx.row_pos, ctx.row_slot,
             ctx.cache.slot_len if ctx.prefill else None, cache if writes_cache else None,
-            group.table, group.page_size, group.ring, want_rows=whole)
+            group.table, group.page_size, group.ring, want_rows=whole,
+            cache_t=cache_t if writes_cache else None)
         if whole:
             if writes_cache:
                 ctx.exchange[("latent_rows", line)] = (c, kr)
@@ -120,7 +130,7 @@ class LatentAttention(Mixer):
             o = ops.latent_gate(a, y, self.gate_off, H, dv, P)
         else:
             longest = min(ctx.max_len, window) if window else ctx.max_len
-            nsplit = ops.latent_decode_splits(y.shape[0], H, longest)
+            nsplit = ops.latent_decode_splits(y.shape[0], H, longest, mfma=cache_t is not None)
             if ctx.prefill:
                 # every row is a token of its own over the cache: it sees the keys up to its position
                 slots, lens, more = ctx.row_slot, ctx.row_pos, 1
@@ -128,5 +138,5 @@ class LatentAttention(Mixer):
                 slots, lens, more = ctx.seq_slot, ctx.seq_len, 0
             o = ops.latent_attn_decode(y, self.w_uk, self.w_uv, self.gate_off, cache, group.table,
                                        group.page_size, group.ring, slots, lens, more, H, dn, dr,
-                                       R, dv, self.scale, window, nsplit)
+                                       R, dv, self.scale, window, nsplit, cache_t)
         return ops.linear(o, self.w_o)

@@ -15,8 +15,8 @@ import torch
 F64 = torch.float64
 
 
-def embed(tokens, table):
-    return table[tokens.long()].to(torch.float32)
+def embed(tokens, table, scale=1.0):
+    return table[tokens.long()].to(torch.float32) * scale
 
 
 def add_rmsnorm(x, delta, weight, eps, out_dtype, row_idx=None):
