@@ -244,9 +244,10 @@ int illm_latent_pack(const void* y, int dt, int ncols, const void* kvu, const vo
 int illm_latent_gate(const void* attn, const void* y, int dt, int ncols, int gate_off, void* out,
                      int T, int H, int dv, int P, void* stream);
 
-// qa[b, h] = [W_uk,h^T q_h (R) | rotated part of q_h (dr)] as float32 [B, H, R + dr], q from y.
-int illm_latent_absorb_q(const void* y, int dt, int ncols, const void* wuk, int w_dt, float* qa,
-                         int B, int H, int dn, int dr, int R, void* stream);
+// qa[b, h] = [W_uk,h^T q_h (R) | rotated part of q_h (dr)] as [B, H, R + dr] of qa_dt (float32
+// sums), q from y.
+int illm_latent_absorb_q(const void* y, int dt, int ncols, const void* wuk, int w_dt, void* qa,
+                         int qa_dt, int B, int H, int dn, int dr, int R, void* stream);
 
 // One token per sequence over the latent cache: scores qa[b, h] . cache row, softmax over the
 // keys the token sees (all, or the last `window`), sums of latent rows.  Token b sees
@@ -258,8 +259,9 @@ int illm_latent_attn_decode(const float* qa, const void* cache, int dt, const in
                             int H, int R, int dr, float scale, int window, void* stream);
 
 // The same on the matrix cores for a bfloat16 cache with R % 16 == 0, (R + dr) % 8 == 0 and pages of
-// a multiple of 32 rows; cache_t: the transposed copy that illm_latent_rope_store keeps.
-int illm_latent_attn_decode_mfma(const float* qa, const void* cache, const void* cache_t,
+// a multiple of 32 rows; cache_t: the transposed copy that illm_latent_rope_store keeps; qa in
+// bfloat16.
+int illm_latent_attn_decode_mfma(const void* qa, const void* cache, const void* cache_t,
                                  const int32_t* page_table, int table_stride, int page_size,
                                  int ring, const int32_t* seq_slot, const int32_t* seq_len,
                                  int len_more, float* partial, int nsplit, int B, int H, int R,

@@ -173,20 +173,20 @@ extern "C" int illm_latent_gate(const void* attn, const void* y, int dt, int nco
 // qa[b, h] = [sum_d q[b, h, d] W_uk[h dn + d, :] (R) | q[b, h, dn:] (dr)], float32.  grid (B, H).
 __global__ void __launch_bounds__(256)
 latent_absorb_q_kernel(const void* __restrict__ y, int dt, int ncols, const void* __restrict__ wuk,
-                       int w_dt, float* __restrict__ qa, int H, int dn, int dr, int R) {
+                       int w_dt, void* __restrict__ qa, int qa_dt, int H, int dn, int dr, int R) {
     extern __shared__ float qs[];
     const int b = blockIdx.x, h = blockIdx.y;
     const size_t src = (size_t)b * ncols + (size_t)h * (dn + dr);
     for (int d = threadIdx.x; d < dn + dr; d += blockDim.x) qs[d] = ld_f(y, dt, src + d);
     __syncthreads();
-    float* dst = qa + ((size_t)b * H + h) * (size_t)(R + dr);
+    const size_t dst = ((size_t)b * H + h) * (size_t)(R + dr);
     for (int r = threadIdx.x; r < R; r += blockDim.x) {
         float acc = 0.f;
 #pragma unroll 8
         for (int d = 0; d < dn; ++d) acc += qs[d] * ld_f(wuk, w_dt, ((size_t)h * dn + d) * R + r);
-        dst[r] = acc;
+        st_f(qa, qa_dt, dst + r, acc);
     }
-    for (int e = threadIdx.x; e < dr; e += blockDim.x) dst[R + e] = qs[dn + e];
+    for (int e = threadIdx.x; e < dr; e += blockDim.x) st_f(qa, qa_dt, dst + R + e, qs[dn + e]);
 }
 
 // The same for bfloat16 W_uk with R % 8 == 0 and R <= 512: a thread holds 8 neighbouring latent
@@ -194,8 +194,8 @@ latent_absorb_q_kernel(const void* __restrict__ y, int dt, int ncols, const void
 // sums are added through LDS in group order.
 __global__ void __launch_bounds__(256)
 latent_absorb_q_bf16_kernel(const void* __restrict__ y, int dt, int ncols,
-                            const bf16_t* __restrict__ wuk, float* __restrict__ qa, int H, int dn,
-                            int dr, int R) {
+                            const bf16_t* __restrict__ wuk, void* __restrict__ qa, int qa_dt, int H,
+                            int dn, int dr, int R) {
     extern __shared__ float sm[];
     float* qs = sm;                       // [dn + dr]
     float* part = sm + dn + dr;           // [groups][R]
@@ -225,19 +225,20 @@ latent_absorb_q_bf16_kernel(const void* __restrict__ y, int dt, int ncols,
         for (int i = 0; i < 8; ++i) part[(size_t)g * R + c * 8 + i] = acc[i];
     }
     __syncthreads();
-    float* dst = qa + ((size_t)b * H + h) * (size_t)(R + dr);
+    const size_t dst = ((size_t)b * H + h) * (size_t)(R + dr);
     for (int r = threadIdx.x; r < R; r += 256) {
         float a = 0.f;
         for (int gg = 0; gg < groups; ++gg) a += part[(size_t)gg * R + r];
-        dst[r] = a;
+        st_f(qa, qa_dt, dst + r, a);
     }
-    for (int e = threadIdx.x; e < dr; e += 256) dst[R + e] = qs[dn + e];
+    for (int e = threadIdx.x; e < dr; e += 256) st_f(qa, qa_dt, dst + R + e, qs[dn + e]);
 }
 
 extern "C" int illm_latent_absorb_q(const void* y, int dt, int ncols, const void* wuk, int w_dt,
-                                    float* qa, int B, int H, int dn, int dr, int R, void* stream) {
+                                    void* qa, int qa_dt, int B, int H, int dn, int dr, int R,
+                                    void* stream) {
     if (B < 0 || H <= 0 || H > 65535 || dn < 0 || dr < 0 || R <= 0 || !illm_dtype_ok(dt) ||
-        !illm_dtype_ok(w_dt) || ncols < H * (dn + dr))
+        !illm_dtype_ok(w_dt) || !illm_dtype_ok(qa_dt) || ncols < H * (dn + dr))
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
     if (w_dt == ILLM_BF16 && R % 8 == 0 && R <= 512 && R >= 8) {
@@ -245,12 +246,12 @@ extern "C" int illm_latent_absorb_q(const void* y, int dt, int ncols, const void
         const size_t smem = ((size_t)(dn + dr) + (size_t)groups * R) * sizeof(float);
         if (smem <= 48 * 1024) {
             hipLaunchKernelGGL(latent_absorb_q_bf16_kernel, dim3(B, H), dim3(256), smem,
-                               (hipStream_t)stream, y, dt, ncols, (const bf16_t*)wuk, qa, H, dn, dr, R);
+                               (hipStream_t)stream, y, dt, ncols, (const bf16_t*)wuk, qa, qa_dt, H, dn, dr, R);
             return illm_launch_status();
         }
     }
     hipLaunchKernelGGL(latent_absorb_q_kernel, dim3(B, H), dim3(256), (size_t)(dn + dr) * sizeof(float),
-                       (hipStream_t)stream, y, dt, ncols, wuk, w_dt, qa, H, dn, dr, R);
+                       (hipStream_t)stream, y, dt, ncols, wuk, w_dt, qa, qa_dt, H, dn, dr, R);
     return illm_launch_status();
 }
 
@@ -457,8 +458,8 @@ extern "C" int illm_latent_attn_decode(const float* qa, const void* cache, int d
 // a multiple of 32 rows), with a second copy of the latent rows laid out [page][dim][row]
 // (`cache_t`).  A block is one wave: a group of 16 heads, one range of keys, 32 keys at a time.
 // Scores: MFMA 16x16x32 with 16 keys as the A operand (8 neighbouring dims of a cache row, read in
-// operand order straight from memory) and the 16 heads' queries as the B operand (bfloat16, in
-// LDS): lane (r, q) = (lane % 16, lane / 16) is left with head r's scores of keys 4 q .. 4 q + 3 of
+// operand order straight from memory) and the 16 heads' queries as the B operand (bfloat16, read
+// the same way; they stay in the cache): lane (r, q) = (lane % 16, lane / 16) is left with head r's scores of keys 4 q .. 4 q + 3 of
 // either half of the 32.  Those 8 weights are the B operand of the second product as they stand:
 // its contraction takes the keys in that order, and the A operand, 16 latent dims by these 8 keys,
 // is two 8-byte loads from the transposed copy.  Keys that are not seen get weight 0 and their
@@ -469,16 +470,14 @@ typedef float la_f32x4_t __attribute__((ext_vector_type(4)));
 
 template <int RT>
 __global__ void __launch_bounds__(64)
-latent_decode_mfma_kernel(const float* __restrict__ qa, const bf16_t* __restrict__ cache,
+latent_decode_mfma_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restrict__ cache,
                           const bf16_t* __restrict__ cache_t,
                           const int32_t* __restrict__ page_table, int table_stride, int page_size,
                           int ring, const int32_t* __restrict__ seq_slot,
                           const int32_t* __restrict__ seq_len, int len_more,
                           float* __restrict__ partial, int nsplit, int H, int R, int dr, float scale,
                           int window) {
-    extern __shared__ uint4 qs_raw[];
-    bf16_t* qs = (bf16_t*)qs_raw;                      // [16][D + 8]
-    const int D = R + dr, QS = D + 8;
+    const int D = R + dr;
     const int b = blockIdx.x, split = blockIdx.y, h0 = blockIdx.z * 16;
     const int lane = threadIdx.x, r = lane & 15, q = lane >> 4;
     const int len = seq_len[b] + len_more, slot = seq_slot[b];
@@ -487,11 +486,8 @@ latent_decode_mfma_kernel(const float* __restrict__ qa, const bf16_t* __restrict
     const int per = (tile1 - tile0 + nsplit - 1) / nsplit;
     const int ta = tile0 + split * per;
     const int tb = ta + per < tile1 ? ta + per : tile1;
-    for (int e = lane; e < 16 * D; e += 64) {
-        const int hh = e / D, d = e - hh * D;
-        qs[hh * QS + d] = f32_to_bf16(h0 + hh < H ? qa[((size_t)b * H + h0 + hh) * D + d] : 0.f);
-    }
-    __syncthreads();
+    // the lane's query row (heads beyond the last read the last one's; their results are dropped)
+    const bf16_t* qp = qa + ((size_t)b * H + (h0 + r < H ? h0 + r : H - 1)) * D + 8 * q;
     la_f32x4_t o[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) o[rt] = (la_f32x4_t){0.f, 0.f, 0.f, 0.f};
@@ -510,7 +506,7 @@ latent_decode_mfma_kernel(const float* __restrict__ qa, const bf16_t* __restrict
         for (int d0 = 0; d0 < D; d0 += 32) {
             la_bf16x8_t qv = zero8, ka = zero8, kb = zero8;
             if (d0 + 8 * q < D) {
-                qv = *(const la_bf16x8_t*)(qs + r * QS + d0 + 8 * q);
+                qv = *(const la_bf16x8_t*)(qp + d0);
                 ka = *(const la_bf16x8_t*)(kp0 + d0);
                 kb = *(const la_bf16x8_t*)(kp1 + d0);
             }
@@ -580,7 +576,7 @@ latent_decode_mfma_kernel(const float* __restrict__ qa, const bf16_t* __restrict
     }
 }
 
-extern "C" int illm_latent_attn_decode_mfma(const float* qa, const void* cache, const void* cache_t,
+extern "C" int illm_latent_attn_decode_mfma(const void* qa, const void* cache, const void* cache_t,
                                             const int32_t* page_table, int table_stride,
                                             int page_size, int ring, const int32_t* seq_slot,
                                             const int32_t* seq_len, int len_more, float* partial,
@@ -593,12 +589,11 @@ extern "C" int illm_latent_attn_decode_mfma(const float* qa, const void* cache, 
     if (B == 0) return ILLM_OK;
     const int groups = (H + 15) / 16;
     if (groups > 65535) return ILLM_ERR_ARG;
-    const size_t smem = (size_t)16 * (R + dr + 8) * sizeof(bf16_t);
     const dim3 grid(B, nsplit, groups);
     hipStream_t st = (hipStream_t)stream;
 #define GO(RT_)                                                                                   \
-    hipLaunchKernelGGL((latent_decode_mfma_kernel<RT_>), grid, dim3(64), smem, st, qa,             \
-                       (const bf16_t*)cache, (const bf16_t*)cache_t, page_table, table_stride,     \
+    hipLaunchKernelGGL((latent_decode_mfma_kernel<RT_>), grid, dim3(64), 0, st,                    \
+                       (const bf16_t*)qa, (const bf16_t*)cache, (const bf16_t*)cache_t, page_table, table_stride,     \
                        page_size, ring, seq_slot, seq_len, len_more, partial, nsplit, H, R, dr,    \
                        scale, window)
     if (R <= 64) GO(4);
@@ -647,20 +642,31 @@ latent_merge_up_kernel(const float* __restrict__ partial, int nsplit, const void
     if (w_dt == ILLM_BF16 && R % 8 == 0) {
         // 16-byte loads: a lane takes 8 neighbouring latent dims of a row of W_uv
         const bf16_t* wp = (const bf16_t*)wuv;
-        for (int v = w; v < dv; v += 4) {
-            const size_t wr = ((size_t)h * dv + v) * R;
-            float dot = 0.f;
+        for (int v0 = 4 * w; v0 < dv; v0 += 16) {           // four rows of W_uv in flight a wave
+            float dot[4] = {0.f, 0.f, 0.f, 0.f};
             for (int r = lane * 8; r < R; r += 512) {
-                const uint4 u = *(const uint4*)(wp + wr + r);
-                const uint32_t uw[4] = {u.x, u.y, u.z, u.w};
+                uint4 u[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    dot += __uint_as_float(uw[i] << 16) * ol[r + 2 * i];
-                    dot += __uint_as_float(uw[i] & 0xffff0000u) * ol[r + 2 * i + 1];
+                for (int j = 0; j < 4; ++j) {
+                    const int v = v0 + j < dv ? v0 + j : dv - 1;
+                    u[j] = *(const uint4*)(wp + ((size_t)h * dv + v) * R + r);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t uw[4] = {u[j].x, u[j].y, u[j].z, u[j].w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        dot[j] += __uint_as_float(uw[i] << 16) * ol[r + 2 * i];
+                        dot[j] += __uint_as_float(uw[i] & 0xffff0000u) * ol[r + 2 * i + 1];
+                    }
                 }
             }
-            dot = wave_sum(dot);
-            if (lane == 0) st_f(out, dt, (size_t)b * H * dv + (size_t)h * dv + v, dot * gate);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float d = wave_sum(dot[j]);
+                if (lane == 0 && v0 + j < dv)
+                    st_f(out, dt, (size_t)b * H * dv + (size_t)h * dv + v0 + j, d * gate);
+            }
         }
         return;
     }

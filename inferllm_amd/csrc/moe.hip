@@ -13,28 +13,54 @@
 #define MOE_TILE 8
 
 // ---------------------------------------------------------------- router
-// z[t, e] = sum_k x[t, k] w[e, k] with a float32 matrix of few rows (a router): a wave an output,
-// lanes over K, float32 products and sums in an order fixed by K.  grid (T, ceil(NE / 4)).
+// z[t, e] = sum_k x[t, k] w[e, k] with a float32 matrix of few rows (a router): float32 products
+// and sums.  A wave takes 4 outputs and 8 tokens at a time (a chunk of a row of w serves 8 tokens,
+// a chunk of a token's row 4 outputs), lanes over K; every sum runs over K in the same order
+// whatever its companions.  grid (ceil(T / 8), ceil(NE / 16)).
 __global__ void __launch_bounds__(256)
 few_outputs_f32_kernel(const void* __restrict__ x, int x_dt, const float* __restrict__ w,
-                       float* __restrict__ z, int NE, int K) {
-    const size_t t = blockIdx.x;
-    const int e = blockIdx.y * 4 + wave_index(), lane = threadIdx.x & 63;
-    if (e >= NE) return;
-    const float* wr = w + (size_t)e * K;
-    float acc = 0.f;
-#pragma unroll 4
-    for (int k = lane; k < K; k += 64) acc += ld_f(x, x_dt, t * K + k) * wr[k];
-    acc = wave_sum(acc);
-    if (lane == 0) z[t * NE + e] = acc;
+                       float* __restrict__ z, int T, int NE, int K) {
+    const int t0 = blockIdx.x * 8;
+    const int e0 = (blockIdx.y * 4 + wave_index()) * 4, lane = threadIdx.x & 63;
+    if (e0 >= NE) return;
+    const float* wr[4];
+    size_t xr[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) wr[j] = w + (size_t)(e0 + j < NE ? e0 + j : NE - 1) * K;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xr[i] = (size_t)(t0 + i < T ? t0 + i : T - 1) * K;
+    float acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+#pragma unroll 2
+    for (int k = lane; k < K; k += 64) {
+        float wv[4], xv[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) wv[j] = wr[j][k];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xv[i] = ld_f(x, x_dt, xr[i] + k);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] += xv[i] * wv[j];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float v = wave_sum(acc[i][j]);
+            if (lane == 0 && t0 + i < T && e0 + j < NE) z[(size_t)(t0 + i) * NE + e0 + j] = v;
+        }
 }
 
 extern "C" int illm_few_outputs_f32(const void* x, int x_dt, const float* w, float* z, int T, int NE,
                                     int K, void* stream) {
-    if (T < 0 || NE <= 0 || NE > 65535 * 4 || K <= 0 || !illm_dtype_ok(x_dt)) return ILLM_ERR_ARG;
+    if (T < 0 || NE <= 0 || NE > 65535 * 16 || K <= 0 || !illm_dtype_ok(x_dt)) return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
-    hipLaunchKernelGGL(few_outputs_f32_kernel, dim3(T, (NE + 3) / 4), dim3(256), 0, (hipStream_t)stream,
-                       x, x_dt, w, z, NE, K);
+    hipLaunchKernelGGL(few_outputs_f32_kernel, dim3((T + 7) / 8, (NE + 15) / 16), dim3(256), 0,
+                       (hipStream_t)stream, x, x_dt, w, z, T, NE, K);
     return illm_launch_status();
 }
 
@@ -320,15 +346,25 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __re
             a[nt][mt] = (moe_f32x4_t){0.f, 0.f, 0.f, 0.f};
             g[nt][mt] = a[nt][mt];
         }
+    // the operands of the next 32 k are asked for before this step's products are issued
+    moe_bf16x8_t w0[NT], w1[NT], x[MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        w0[nt] = *(const moe_bf16x8_t*)(wa[nt]);
+        if (GATED) w1[nt] = *(const moe_bf16x8_t*)(wa[nt] + up);
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) x[mt] = *(const moe_bf16x8_t*)(xp[mt]);
     for (int k = 0; k < K; k += 32) {
-        moe_bf16x8_t w0[NT], w1[NT], x[MT];
+        moe_bf16x8_t w0n[NT], w1n[NT], xn[MT];
+        const int kn = k + 32 < K ? k + 32 : k;            // the last step loads its own again
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            w0[nt] = *(const moe_bf16x8_t*)(wa[nt] + k);
-            if (GATED) w1[nt] = *(const moe_bf16x8_t*)(wa[nt] + up + k);
+            w0n[nt] = *(const moe_bf16x8_t*)(wa[nt] + kn);
+            if (GATED) w1n[nt] = *(const moe_bf16x8_t*)(wa[nt] + up + kn);
         }
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) x[mt] = *(const moe_bf16x8_t*)(xp[mt] + k);
+        for (int mt = 0; mt < MT; ++mt) xn[mt] = *(const moe_bf16x8_t*)(xp[mt] + kn);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -337,6 +373,13 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __re
                 if (GATED)
                     g[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[nt], x[mt], g[nt][mt], 0, 0, 0);
             }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            w0[nt] = w0n[nt];
+            if (GATED) w1[nt] = w1n[nt];
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) x[mt] = xn[mt];
     }
     // a[nt][mt][i] belongs to the pair of row mt * 16 + r and column n0 + 16 nt + 4 q + i
 #pragma unroll
@@ -375,7 +418,10 @@ extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int g
                            (const bf16_t*)X, x_div, (const bf16_t*)W, order, tiles, max_tiles,     \
                            (bf16_t*)Y, N, K);                                                      \
     } while (0)
-    if (tile_rows == 16) { if (gated) GO(1, 4, true); else GO(1, 4, false); }
+    if (tile_rows == 16 && (long)max_tiles * ((N + 255) / 256) < 512) {
+        // few tiles (single tokens): 16 columns a wave, so that more waves share the reading
+        if (gated) GO(1, 1, true); else GO(1, 1, false);
+    } else if (tile_rows == 16) { if (gated) GO(1, 4, true); else GO(1, 4, false); }
     else if (tile_rows == 32) { if (gated) GO(2, 4, true); else GO(2, 4, false); }
     else { if (gated) GO(4, 2, true); else GO(4, 4, false); }
 #undef GO

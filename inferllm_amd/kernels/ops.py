@@ -1138,9 +1138,11 @@ def latent_attn_decode(y: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor, 
     _need(w_uk.shape == (H * dn, R) and w_uv.shape == (H * dv, R), "latent_attn_decode: W_uk / W_uv")
     _need(cache.dim() == 3 and cache.shape[1:] == (page_size, R + dr) and cache.dtype == y.dtype,
           "latent_attn_decode: cache shape or dtype")
-    qa = torch.empty((B, H, R + dr), dtype=torch.float32, device=y.device)
+    # the matrix-core kernel takes the queries in bfloat16 (they are an operand of its product)
+    qa = torch.empty((B, H, R + dr), dtype=torch.bfloat16 if cache_t is not None else torch.float32,
+                     device=y.device)
     _check(_lib().illm_latent_absorb_q(_p(y), _code(y), y.shape[1], _p(w_uk), _code(w_uk), _p(qa),
-                                       B, H, dn, dr, R, _stream()), "latent_absorb_q")
+                                       _code(qa), B, H, dn, dr, R, _stream()), "latent_absorb_q")
     partial = torch.empty((B, H, nsplit, R + 2), dtype=torch.float32, device=y.device)
     if cache_t is not None:
         _need(latent_decode_mfma_fits(cache, cache_t, R, dr, page_size) and
@@ -1191,8 +1193,10 @@ def moe_route(z: torch.Tensor, correction: Optional[torch.Tensor], top: int):
     return idx, wt
 
 
-MOE_MFMA_FROM = 8        # (token, choice) pairs an expert on average from which the experts' products
-                         # run on the matrix cores (below: a wave a column, lanes over K)
+MOE_MFMA_FROM = 0        # (token, choice) pairs an expert on average from which the experts' products
+                         # run on the matrix cores where the shape allows (measured on MI355X, 64
+                         # experts of 1408 x 2048, 6 of them a token: a wave a column with lanes over
+                         # K took 253 + 166 us for 64 tokens, bound by its sums across lanes)
 
 
 def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
