@@ -604,8 +604,9 @@ extern "C" int illm_latent_attn_decode_mfma(const void* qa, const void* cache, c
     return illm_launch_status();
 }
 
-// grid (B, H): combine the splits, multiply the combined latent sum by W_uv's rows of the head
-// (a wave a value dim, lanes over the latent dims) and by the head's output gate.
+// grid (B, H, chunks of 32 value dims): combine the splits, multiply the combined latent sum by
+// W_uv's rows of the head (a wave a value dim, lanes over the latent dims) and by the head's
+// output gate.  Every chunk's block combines the splits for itself.
 __global__ void __launch_bounds__(256)
 latent_merge_up_kernel(const float* __restrict__ partial, int nsplit, const void* __restrict__ wuv,
                        int w_dt, const void* __restrict__ y, int dt, int ncols, int gate_off,
@@ -642,13 +643,14 @@ latent_merge_up_kernel(const float* __restrict__ partial, int nsplit, const void
     if (w_dt == ILLM_BF16 && R % 8 == 0) {
         // 16-byte loads: a lane takes 8 neighbouring latent dims of a row of W_uv
         const bf16_t* wp = (const bf16_t*)wuv;
-        for (int v0 = 4 * w; v0 < dv; v0 += 16) {           // four rows of W_uv in flight a wave
+        const int v_end = min(dv, (int)(blockIdx.z + 1) * 32);
+        for (int v0 = blockIdx.z * 32 + 4 * w; v0 < v_end; v0 += 16) {   // four rows of W_uv in flight a wave
             float dot[4] = {0.f, 0.f, 0.f, 0.f};
             for (int r = lane * 8; r < R; r += 512) {
                 uint4 u[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int v = v0 + j < dv ? v0 + j : dv - 1;
+                    const int v = v0 + j < v_end ? v0 + j : v_end - 1;
                     u[j] = *(const uint4*)(wp + ((size_t)h * dv + v) * R + r);
                 }
 #pragma unroll
@@ -664,13 +666,14 @@ latent_merge_up_kernel(const float* __restrict__ partial, int nsplit, const void
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const float d = wave_sum(dot[j]);
-                if (lane == 0 && v0 + j < dv)
+                if (lane == 0 && v0 + j < v_end)
                     st_f(out, dt, (size_t)b * H * dv + (size_t)h * dv + v0 + j, d * gate);
             }
         }
         return;
     }
-    for (int v = w; v < dv; v += 4) {
+    const int v_hi = min(dv, (int)(blockIdx.z + 1) * 32);
+    for (int v = blockIdx.z * 32 + w; v < v_hi; v += 4) {
         const size_t wr = ((size_t)h * dv + v) * R;
         float dot = 0.f;
         for (int r = lane; r < R; r += 64) dot += ld_f(wuv, w_dt, wr + r) * ol[r];
@@ -686,7 +689,8 @@ extern "C" int illm_latent_merge_up(const float* partial, int nsplit, const void
         !illm_dtype_ok(w_dt) || gate_off < 0 || gate_off + H > ncols)
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
-    hipLaunchKernelGGL(latent_merge_up_kernel, dim3(B, H), dim3(256), (size_t)(R + nsplit) * sizeof(float),
+    if ((dv + 31) / 32 > 65535) return ILLM_ERR_ARG;
+    hipLaunchKernelGGL(latent_merge_up_kernel, dim3(B, H, (dv + 31) / 32), dim3(256), (size_t)(R + nsplit) * sizeof(float),
                        (hipStream_t)stream, partial, nsplit, wuv, w_dt, y, dt, ncols, gate_off, out,
                        H, R, dv);
     return illm_launch_status();

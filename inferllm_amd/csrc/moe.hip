@@ -17,50 +17,58 @@
 // and sums.  A wave takes 4 outputs and 8 tokens at a time (a chunk of a row of w serves 8 tokens,
 // a chunk of a token's row 4 outputs), lanes over K; every sum runs over K in the same order
 // whatever its companions.  grid (ceil(T / 8), ceil(NE / 16)).
+template <int EW>
 __global__ void __launch_bounds__(256)
 few_outputs_f32_kernel(const void* __restrict__ x, int x_dt, const float* __restrict__ w,
                        float* __restrict__ z, int T, int NE, int K) {
     const int t0 = blockIdx.x * 8;
-    const int e0 = (blockIdx.y * 4 + wave_index()) * 4, lane = threadIdx.x & 63;
+    const int e0 = (blockIdx.y * 4 + wave_index()) * EW, lane = threadIdx.x & 63;
     if (e0 >= NE) return;
-    const float* wr[4];
+    const int nt = T - t0 < 8 ? T - t0 : 8;
+    const float* wr[EW];
     size_t xr[8];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) wr[j] = w + (size_t)(e0 + j < NE ? e0 + j : NE - 1) * K;
+    for (int j = 0; j < EW; ++j) wr[j] = w + (size_t)(e0 + j < NE ? e0 + j : NE - 1) * K;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) xr[i] = (size_t)(t0 + i < T ? t0 + i : T - 1) * K;
-    float acc[8][4];
+    for (int i = 0; i < 8; ++i) xr[i] = (size_t)(i < nt ? t0 + i : t0) * K;
+    float acc[8][EW];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+        for (int j = 0; j < EW; ++j) acc[i][j] = 0.f;
 #pragma unroll 2
     for (int k = lane; k < K; k += 64) {
-        float wv[4], xv[8];
+        float wv[EW], xv[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) wv[j] = wr[j][k];
+        for (int j = 0; j < EW; ++j) wv[j] = wr[j][k];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) xv[i] = ld_f(x, x_dt, xr[i] + k);
+        for (int i = 0; i < 8; ++i) xv[i] = i < nt ? ld_f(x, x_dt, xr[i] + k) : 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] += xv[i] * wv[j];
+            for (int j = 0; j < EW; ++j) acc[i][j] += xv[i] * wv[j];
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 8; ++i) {
+        if (i >= nt) continue;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < EW; ++j) {
             const float v = wave_sum(acc[i][j]);
-            if (lane == 0 && t0 + i < T && e0 + j < NE) z[(size_t)(t0 + i) * NE + e0 + j] = v;
+            if (lane == 0 && e0 + j < NE) z[(size_t)(t0 + i) * NE + e0 + j] = v;
         }
+    }
 }
 
 extern "C" int illm_few_outputs_f32(const void* x, int x_dt, const float* w, float* z, int T, int NE,
                                     int K, void* stream) {
-    if (T < 0 || NE <= 0 || NE > 65535 * 16 || K <= 0 || !illm_dtype_ok(x_dt)) return ILLM_ERR_ARG;
+    if (T < 0 || NE <= 0 || NE > 65535 * 4 || K <= 0 || !illm_dtype_ok(x_dt)) return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
-    hipLaunchKernelGGL(few_outputs_f32_kernel, dim3((T + 7) / 8, (NE + 15) / 16), dim3(256), 0,
-                       (hipStream_t)stream, x, x_dt, w, z, T, NE, K);
+    if (T <= 16)        // few tokens: an output a wave, so that more waves share the reading
+        hipLaunchKernelGGL(few_outputs_f32_kernel<1>, dim3((T + 7) / 8, (NE + 3) / 4), dim3(256), 0,
+                           (hipStream_t)stream, x, x_dt, w, z, T, NE, K);
+    else
+        hipLaunchKernelGGL(few_outputs_f32_kernel<4>, dim3((T + 7) / 8, (NE + 15) / 16), dim3(256), 0,
+                           (hipStream_t)stream, x, x_dt, w, z, T, NE, K);
     return illm_launch_status();
 }
 
@@ -309,7 +317,7 @@ extern "C" int illm_moe_rows(const void* X, int x_div, const void* W, int dt, in
 typedef __bf16 moe_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float moe_f32x4_t __attribute__((ext_vector_type(4)));
 
-template <int MT, int NT, bool GATED>
+template <int MT, int NT, bool GATED, bool AHEAD>
 __global__ void __launch_bounds__(256)
 moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __restrict__ W,
                      const int32_t* __restrict__ order, const int32_t* __restrict__ tiles,
@@ -358,13 +366,25 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __re
     for (int k = 0; k < K; k += 32) {
         moe_bf16x8_t w0n[NT], w1n[NT], xn[MT];
         const int kn = k + 32 < K ? k + 32 : k;            // the last step loads its own again
+        if (!AHEAD && k > 0) {
+            // (many accumulators: no second set of operands; other waves hide the loads)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            w0n[nt] = *(const moe_bf16x8_t*)(wa[nt] + kn);
-            if (GATED) w1n[nt] = *(const moe_bf16x8_t*)(wa[nt] + up + kn);
+            for (int nt = 0; nt < NT; ++nt) {
+                w0[nt] = *(const moe_bf16x8_t*)(wa[nt] + k);
+                if (GATED) w1[nt] = *(const moe_bf16x8_t*)(wa[nt] + up + k);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) x[mt] = *(const moe_bf16x8_t*)(xp[mt] + k);
         }
+        if (AHEAD) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xn[mt] = *(const moe_bf16x8_t*)(xp[mt] + kn);
+            for (int nt = 0; nt < NT; ++nt) {
+                w0n[nt] = *(const moe_bf16x8_t*)(wa[nt] + kn);
+                if (GATED) w1n[nt] = *(const moe_bf16x8_t*)(wa[nt] + up + kn);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) xn[mt] = *(const moe_bf16x8_t*)(xp[mt] + kn);
+        }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -373,13 +393,15 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __re
                 if (GATED)
                     g[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[nt], x[mt], g[nt][mt], 0, 0, 0);
             }
+        if (AHEAD) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            w0[nt] = w0n[nt];
-            if (GATED) w1[nt] = w1n[nt];
+            for (int nt = 0; nt < NT; ++nt) {
+                w0[nt] = w0n[nt];
+                if (GATED) w1[nt] = w1n[nt];
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) x[mt] = xn[mt];
         }
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) x[mt] = xn[mt];
     }
     // a[nt][mt][i] belongs to the pair of row mt * 16 + r and column n0 + 16 nt + 4 q + i
 #pragma unroll
@@ -414,7 +436,7 @@ extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int g
     do {                                                                                           \
         const dim3 grid(max_tiles, (N + 64 * NT_ - 1) / (64 * NT_));                               \
         if (grid.y > 65535) return ILLM_ERR_ARG;                                                   \
-        hipLaunchKernelGGL((moe_rows_mfma_kernel<MT_, NT_, G_>), grid, dim3(256), 0, st,           \
+        hipLaunchKernelGGL((moe_rows_mfma_kernel<MT_, NT_, G_, (MT_ * NT_ <= 16)>), grid, dim3(256), 0, st, \
                            (const bf16_t*)X, x_div, (const bf16_t*)W, order, tiles, max_tiles,     \
                            (bf16_t*)Y, N, K);                                                      \
     } while (0)
@@ -423,14 +445,15 @@ extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int g
         if (gated) GO(1, 1, true); else GO(1, 1, false);
     } else if (tile_rows == 16) { if (gated) GO(1, 4, true); else GO(1, 4, false); }
     else if (tile_rows == 32) { if (gated) GO(2, 4, true); else GO(2, 4, false); }
-    else { if (gated) GO(4, 2, true); else GO(4, 4, false); }
+    else { if (gated) GO(4, 2, true); else GO(4, 4, false); }    // wider column blocks measured slower
 #undef GO
     return illm_launch_status();
 }
 
 // ---------------------------------------------------------------- weighted sum
-// One block per token: out[t] = sum_k wt[t, k] * (idx[t, k] < NEr ? Y[t top + k] : h[t])
-//                               (+ sigmoid(h[t] . sg) * shared[t]), float32.
+// grid (tokens, chunks of 1024 columns): out[t] = sum_k wt[t, k] * (idx[t, k] < NEr ? Y[t top + k] : h[t])
+//                                         (+ sigmoid(h[t] . sg) * shared[t]), float32.
+#define MOE_COMBINE_TOP 16                          // choices held in registers (more: read again)
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const void* __restrict__ h, int dt, const int32_t* __restrict__ idx,
                    const float* __restrict__ wt, const void* __restrict__ Y,
@@ -438,6 +461,13 @@ moe_combine_kernel(const void* __restrict__ h, int dt, const int32_t* __restrict
                    float* __restrict__ out, int E, int top, int NEr) {
     __shared__ float red[16];
     const size_t t = blockIdx.x;
+    int ce[MOE_COMBINE_TOP];
+    float cw[MOE_COMBINE_TOP];
+#pragma unroll
+    for (int k = 0; k < MOE_COMBINE_TOP; ++k) {
+        ce[k] = k < top ? idx[t * top + k] : 0;
+        cw[k] = k < top ? wt[t * top + k] : 0.f;
+    }
     float gate = 0.f;
     if (shared) {
         gate = 1.f;
@@ -448,12 +478,23 @@ moe_combine_kernel(const void* __restrict__ h, int dt, const int32_t* __restrict
             gate = 1.0f / (1.0f + expf(-d));
         }
     }
-    for (int i = threadIdx.x; i < E; i += blockDim.x) {
+    const int i_end = min(E, (int)(blockIdx.y + 1) * 1024);
+    for (int i = blockIdx.y * 1024 + threadIdx.x; i < i_end; i += 256) {
+        const float hv = ld_f(h, dt, t * E + i);
         float acc = 0.f;
-        for (int k = 0; k < top; ++k) {
-            const int e = idx[t * top + k];
-            const float v = e < NEr ? ld_f(Y, dt, (t * top + k) * E + i) : ld_f(h, dt, t * E + i);
-            acc += wt[t * top + k] * v;
+        if (top <= MOE_COMBINE_TOP) {
+            float v[MOE_COMBINE_TOP];
+#pragma unroll
+            for (int k = 0; k < MOE_COMBINE_TOP; ++k)
+                v[k] = k < top && ce[k] < NEr ? ld_f(Y, dt, (t * top + k) * E + i) : hv;
+#pragma unroll
+            for (int k = 0; k < MOE_COMBINE_TOP; ++k)
+                if (k < top) acc += cw[k] * v[k];
+        } else {
+            for (int k = 0; k < top; ++k) {
+                const int e = idx[t * top + k];
+                acc += wt[t * top + k] * (e < NEr ? ld_f(Y, dt, (t * top + k) * E + i) : hv);
+            }
         }
         if (shared) acc += gate * ld_f(shared, dt, t * E + i);
         out[t * E + i] = acc;
@@ -463,10 +504,11 @@ moe_combine_kernel(const void* __restrict__ h, int dt, const int32_t* __restrict
 extern "C" int illm_moe_combine(const void* h, int dt, const int32_t* idx, const float* wt,
                                 const void* Y, const void* shared, const void* sg, int sg_dt,
                                 float* out, int T, int E, int top, int NEr, void* stream) {
-    if (T < 0 || E <= 0 || top <= 0 || !illm_dtype_ok(dt) || (sg && !illm_dtype_ok(sg_dt)))
+    if (T < 0 || E <= 0 || top <= 0 || !illm_dtype_ok(dt) || (sg && !illm_dtype_ok(sg_dt)) ||
+        (E + 1023) / 1024 > 65535)
         return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, h, dt, idx,
-                       wt, Y, shared, sg, sg_dt, out, E, top, NEr);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(T, (E + 1023) / 1024), dim3(256), 0, (hipStream_t)stream,
+                       h, dt, idx, wt, Y, shared, sg, sg_dt, out, E, top, NEr);
     return illm_launch_status();
 }
