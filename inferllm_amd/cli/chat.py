@@ -45,7 +45,7 @@ def build_parser() -> argparse.ArgumentParser:
                     help="compute type (default: bfloat16)")
     ap.add_argument("-g", dest="device", default="GPU", help="compute device type: GPU (CPU is refused)")
     ap.add_argument("--type", dest="mtype", default=None,
-                    help="model type name; must agree with config.json if given (llama, llama2)")
+                    help="model type name; must agree with config.json if given (llama, llama2, rabapel)")
     ap.add_argument("--mmap", action="store_true",
                     help="accepted for compatibility; safetensors files are always memory-mapped")
     ap.add_argument("-n", "--n_predict", type=int, default=128, help="new tokens to predict (default: 128)")

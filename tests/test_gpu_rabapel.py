@@ -217,6 +217,64 @@ def test_greedy_generation_through_the_engine(tmp_path_factory):
     eng.cache.check()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_of_many_short_requests(tmp_path, dtype):
+    """`bin/trace_run` on a Rabapel folder: fourteen requests of 1 to 75 tokens in one batch, then
+    decoded together while the shorter ones end, with --max-tokens the tokens themselves (every
+    request holds a partly filled page on top of that)."""
+    from test_gpu_trace import replay
+    d = write_model(tmp_path, MIXED, seed=21, dtype=STORE[dtype])
+    w = weights64(d)
+    lens = [1, 2, 3, 5, 8, 13, 21, 34, 55, 75, 65, 64, 63, 4]
+    reqs = [random_ids(n + 2 + i % 3, MIXED["vocab"], 50 + i) for i, n in enumerate(lens)]
+    plain = [P.forward(MIXED, w, r) for r in reqs]
+    steps = [{"step": 0, "entries": [{"id": f"r{i}", "tokens": r[:lens[i]], "want": [lens[i] - 1]}
+                                     for i, r in enumerate(reqs)], "end": []}]
+    expect = {0: torch.cat([plain[i][lens[i] - 1:lens[i]] for i in range(len(reqs))])}
+    at, live, n = list(lens), list(range(len(reqs))), 1
+    while live:
+        ends = [i for i in live if at[i] == len(reqs[i]) - 1]
+        steps.append({"step": n, "entries": [{"id": f"r{i}", "tokens": [reqs[i][at[i]]], "want": [0]} for i in live],
+                      "end": [f"r{i}" for i in ends]})
+        expect[n] = torch.cat([plain[i][at[i]:at[i] + 1] for i in live])
+        n += 1
+        for i in live:
+            at[i] += 1
+        live = [i for i in live if i not in ends]
+    got = replay(d, dtype, str(tmp_path / "out"), sum(len(r) for r in reqs), steps)
+    for s_ in sorted(expect):
+        close(torch.from_numpy(got[s_].copy()), expect[s_], dtype, f"step {s_}")
+
+
+def test_command_line_and_a_conversation(tmp_path):
+    """`bin/chat` on a Rabapel folder with token-id prompts, greedy: the plain model's tokens; and
+    `Engine.session`: the turns of a conversation go on from the slot's cache by several tokens."""
+    import os
+    import subprocess
+    import sys
+    d = write_model(tmp_path, MIXED, seed=17)
+    w = weights64(d)
+    prompts = [random_ids(n, MIXED["vocab"], 9 * n) for n in (6, 2)]
+    ids_file = tmp_path / "prompts.txt"
+    ids_file.write_text("\n".join(" ".join(map(str, p)) for p in prompts) + "\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "chat"), "-m", d, "-d", "float32", "--temp", "0",
+                        "-n", "7", "--prompt-ids-file", str(ids_file), "-c", "64", "--type", "rabapel"],
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr
+    got = [[int(t) for t in line.split()] for line in r.stdout.strip().splitlines()]
+    assert got == [P.generate_greedy(MIXED, w, p, 7) for p in prompts]
+    eng = engine_for(d, "float32")
+    with eng.session(stop_token_ids=[]) as chat:
+        said = list(prompts[0])
+        a1 = chat.say(prompts[0], max_new_tokens=4)
+        assert a1 == P.generate_greedy(MIXED, w, said, 4)
+        turn = random_ids(5, MIXED["vocab"], 77)
+        a2 = chat.say(turn, max_new_tokens=3)
+        # the token that max_new_tokens cut off is fed in front of the next turn
+        assert a2 == P.generate_greedy(MIXED, w, said + a1 + turn, 3)
+
+
 def test_architecture_is_chosen_by_config_and_refuses_what_it_lacks(tmp_path_factory):
     import inferllm_amd as I
     assert "Rabapel" in I.registered_architectures()

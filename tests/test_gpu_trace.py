@@ -111,4 +111,4 @@ def test_a_step_that_wants_nothing_writes_nothing_and_bad_input_fails(tmp_path):
                         "--out", str(tmp_path / "o2"), "--max-tokens", "64"],
                        input=json.dumps({"step": 0, "entries": [{"id": "a", "tokens": list(range(65)), "want": [0]}],
                                          "end": []}) + "\n", capture_output=True, text=True)
-    assert p.returncode != 0 and "cache full" in p.stderr
+    assert p.returncode != 0 and "the limit is 64" in p.stderr
