@@ -368,7 +368,7 @@ latent_decode_kernel(const float* __restrict__ qa, const void* __restrict__ cach
     for (int i = 0; i < HGW; ++i) {
         const int h = h0 + w * HGW + i;
         if (h >= H) continue;
-        float* dst = partial + (((size_t)b * H + h) * nsplit + split) * (size_t)(R + 2);
+        float* dst = partial + (((size_t)b * H + h) * nsplit + split) * (size_t)(R + 4);
 #pragma unroll
         for (int c = 0; c < RC; ++c) {
             const int r = lane + 64 * c;
@@ -502,8 +502,23 @@ latent_decode_mfma_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restric
         const bf16_t* kp0 = cache + ((size_t)phys * page_size + rowb + r) * D + 8 * q;
         const bf16_t* kp1 = kp0 + (size_t)16 * D;
         la_f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0;
-#pragma unroll 6
-        for (int d0 = 0; d0 < D; d0 += 32) {
+        // six steps of 32 dims at a time: all their loads are asked for before the first product
+        int d0 = 0;
+        for (; d0 + 192 <= D; d0 += 192) {
+            la_bf16x8_t qv[6], ka[6], kb[6];
+#pragma unroll
+            for (int u = 0; u < 6; ++u) {
+                qv[u] = *(const la_bf16x8_t*)(qp + d0 + 32 * u);
+                ka[u] = *(const la_bf16x8_t*)(kp0 + d0 + 32 * u);
+                kb[u] = *(const la_bf16x8_t*)(kp1 + d0 + 32 * u);
+            }
+#pragma unroll
+            for (int u = 0; u < 6; ++u) {
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[u], qv[u], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[u], qv[u], s1, 0, 0, 0);
+            }
+        }
+        for (; d0 < D; d0 += 32) {                   // what is left, the last step maybe in part
             la_bf16x8_t qv = zero8, ka = zero8, kb = zero8;
             if (d0 + 8 * q < D) {
                 qv = *(const la_bf16x8_t*)(qp + d0);
@@ -549,27 +564,36 @@ latent_decode_mfma_kernel(const bf16_t* __restrict__ qa, const bf16_t* __restric
         const uint32_t k45 = (ok[4] ? 0xffffu : 0u) | (ok[5] ? 0xffff0000u : 0u);
         const uint32_t k67 = (ok[6] ? 0xffffu : 0u) | (ok[7] ? 0xffff0000u : 0u);
         const bf16_t* tp = cache_t + ((size_t)phys * R + r) * page_size + rowb + 4 * q;
+        constexpr int CH = RT < 8 ? RT : 8;          // row groups whose loads are in flight together
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-            if (rt * 16 < R) {
-                const uint2 c0 = *(const uint2*)(tp + (size_t)rt * 16 * page_size);
-                const uint2 c1 = *(const uint2*)(tp + (size_t)rt * 16 * page_size + 16);
-                uint4 cu;
-                cu.x = c0.x & k01; cu.y = c0.y & k23; cu.z = c1.x & k45; cu.w = c1.y & k67;
-                o[rt][0] *= alpha; o[rt][1] *= alpha; o[rt][2] *= alpha; o[rt][3] *= alpha;
-                o[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const la_bf16x8_t*)&cu, pv, o[rt], 0, 0, 0);
+        for (int r0 = 0; r0 < RT; r0 += CH) {
+            uint2 c0[CH], c1[CH];
+#pragma unroll
+            for (int u = 0; u < CH; ++u) {
+                const int rt = (r0 + u) * 16 < R ? r0 + u : 0;      // beyond R: loaded, not used
+                c0[u] = *(const uint2*)(tp + (size_t)rt * 16 * page_size);
+                c1[u] = *(const uint2*)(tp + (size_t)rt * 16 * page_size + 16);
+            }
+#pragma unroll
+            for (int u = 0; u < CH; ++u) {
+                const int rt = r0 + u;
+                if (rt * 16 < R) {
+                    uint4 cu;
+                    cu.x = c0[u].x & k01; cu.y = c0[u].y & k23; cu.z = c1[u].x & k45; cu.w = c1[u].y & k67;
+                    o[rt][0] *= alpha; o[rt][1] *= alpha; o[rt][2] *= alpha; o[rt][3] *= alpha;
+                    o[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const la_bf16x8_t*)&cu, pv, o[rt], 0, 0, 0);
+                }
             }
         }
     }
     // o[rt][i] = sum of head h0 + r over latent dim 16 rt + 4 q + i
     const int h = h0 + r;
     if (h < H) {
-        float* dst = partial + (((size_t)b * H + h) * nsplit + split) * (size_t)(R + 2);
+        float* dst = partial + (((size_t)b * H + h) * nsplit + split) * (size_t)(R + 4);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             if (rt * 16 < R) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) dst[rt * 16 + 4 * q + i] = o[rt][i];
+                *(la_f32x4_t*)(dst + rt * 16 + 4 * q) = o[rt];       // rows of R + 4 floats: 16-byte aligned
             }
         }
         if (q == 0) { dst[R] = m; dst[R + 1] = l; }
@@ -614,19 +638,19 @@ latent_merge_up_kernel(const float* __restrict__ partial, int nsplit, const void
     extern __shared__ float ol[];                      // [R] combined sums, then [nsplit] weights
     float* ws = ol + R;
     const int b = blockIdx.x, h = blockIdx.y;
-    const float* base = partial + ((size_t)b * H + h) * nsplit * (size_t)(R + 2);
+    const float* base = partial + ((size_t)b * H + h) * nsplit * (size_t)(R + 4);
     const int w = wave_index(), lane = threadIdx.x & 63;
     if (w == 0) {
         // the ranges' (max, weight): lane s holds range s, s + 64, ...; weights exp(m_s - M) / total
         float M = -INFINITY;
-        for (int s = lane; s < nsplit; s += 64) M = fmaxf(M, base[(size_t)s * (R + 2) + R]);
+        for (int s = lane; s < nsplit; s += 64) M = fmaxf(M, base[(size_t)s * (R + 4) + R]);
         M = wave_max(M);
         float tot = 0.f;
         for (int s = lane; s < nsplit; s += 64) {
-            const float ms = base[(size_t)s * (R + 2) + R];
+            const float ms = base[(size_t)s * (R + 4) + R];
             const float e = ms == -INFINITY ? 0.f : expf(ms - M);
             ws[s] = e;
-            tot += base[(size_t)s * (R + 2) + R + 1] * e;
+            tot += base[(size_t)s * (R + 4) + R + 1] * e;
         }
         tot = wave_sum(tot);
         for (int s = lane; s < nsplit; s += 64) ws[s] = ws[s] / tot;
@@ -634,7 +658,7 @@ latent_merge_up_kernel(const float* __restrict__ partial, int nsplit, const void
     __syncthreads();
     for (int r = threadIdx.x; r < R; r += 256) {
         float a = 0.f;
-        for (int s = 0; s < nsplit; ++s) a += base[(size_t)s * (R + 2) + r] * ws[s];
+        for (int s = 0; s < nsplit; ++s) a += base[(size_t)s * (R + 4) + r] * ws[s];
         ol[r] = a;
     }
     __syncthreads();

@@ -17,6 +17,15 @@
 // and sums.  A wave takes 4 outputs and 8 tokens at a time (a chunk of a row of w serves 8 tokens,
 // a chunk of a token's row 4 outputs), lanes over K; every sum runs over K in the same order
 // whatever its companions.  grid (ceil(T / 8), ceil(NE / 16)).
+__device__ __forceinline__ float4 ld4_f32(const void* p, int dt, size_t i) {
+    if (dt == ILLM_BF16) {
+        const uint2 u = *(const uint2*)((const bf16_t*)p + i);
+        return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                           __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+    }
+    return *(const float4*)((const float*)p + i);
+}
+
 template <int EW>
 __global__ void __launch_bounds__(256)
 few_outputs_f32_kernel(const void* __restrict__ x, int x_dt, const float* __restrict__ w,
@@ -36,17 +45,37 @@ few_outputs_f32_kernel(const void* __restrict__ x, int x_dt, const float* __rest
     for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < EW; ++j) acc[i][j] = 0.f;
+    if (K % 4 == 0) {
+        // four neighbouring k a lane: one 16-byte load of w and one of 8 or 16 bytes of x
 #pragma unroll 2
-    for (int k = lane; k < K; k += 64) {
-        float wv[EW], xv[8];
+        for (int k = lane * 4; k < K; k += 256) {
+            float4 wv[EW], xv[8];
 #pragma unroll
-        for (int j = 0; j < EW; ++j) wv[j] = wr[j][k];
+            for (int j = 0; j < EW; ++j) wv[j] = *(const float4*)(wr[j] + k);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) xv[i] = i < nt ? ld_f(x, x_dt, xr[i] + k) : 0.f;
+            for (int i = 0; i < 8; ++i)
+                xv[i] = i < nt ? ld4_f32(x, x_dt, xr[i] + k) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+            for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int j = 0; j < EW; ++j) acc[i][j] += xv[i] * wv[j];
+                for (int j = 0; j < EW; ++j) {
+                    acc[i][j] += xv[i].x * wv[j].x; acc[i][j] += xv[i].y * wv[j].y;
+                    acc[i][j] += xv[i].z * wv[j].z; acc[i][j] += xv[i].w * wv[j].w;
+                }
+        }
+    } else {
+#pragma unroll 4
+        for (int k = lane; k < K; k += 64) {
+            float wv[EW], xv[8];
+#pragma unroll
+            for (int j = 0; j < EW; ++j) wv[j] = wr[j][k];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[i] = i < nt ? ld_f(x, x_dt, xr[i] + k) : 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < EW; ++j) acc[i][j] += xv[i] * wv[j];
+        }
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -317,7 +346,7 @@ extern "C" int illm_moe_rows(const void* X, int x_div, const void* W, int dt, in
 typedef __bf16 moe_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float moe_f32x4_t __attribute__((ext_vector_type(4)));
 
-template <int MT, int NT, bool GATED, bool AHEAD>
+template <int MT, int NT, bool GATED, bool AHEAD, int KU>
 __global__ void __launch_bounds__(256)
 moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __restrict__ W,
                      const int32_t* __restrict__ order, const int32_t* __restrict__ tiles,
@@ -354,53 +383,80 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __re
             a[nt][mt] = (moe_f32x4_t){0.f, 0.f, 0.f, 0.f};
             g[nt][mt] = a[nt][mt];
         }
-    // the operands of the next 32 k are asked for before this step's products are issued
-    moe_bf16x8_t w0[NT], w1[NT], x[MT];
+    if (KU > 1) {
+        // few accumulators (single tokens): KU steps of 32 k at a time, all their loads first
+        for (int k = 0; k < K; k += 32 * KU) {
+            moe_bf16x8_t w0[KU][NT], w1[KU][NT], x[KU][MT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        w0[nt] = *(const moe_bf16x8_t*)(wa[nt]);
-        if (GATED) w1[nt] = *(const moe_bf16x8_t*)(wa[nt] + up);
-    }
+            for (int u = 0; u < KU; ++u) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) x[mt] = *(const moe_bf16x8_t*)(xp[mt]);
-    for (int k = 0; k < K; k += 32) {
-        moe_bf16x8_t w0n[NT], w1n[NT], xn[MT];
-        const int kn = k + 32 < K ? k + 32 : k;            // the last step loads its own again
-        if (!AHEAD && k > 0) {
-            // (many accumulators: no second set of operands; other waves hide the loads)
+                for (int nt = 0; nt < NT; ++nt) {
+                    w0[u][nt] = *(const moe_bf16x8_t*)(wa[nt] + k + 32 * u);
+                    if (GATED) w1[u][nt] = *(const moe_bf16x8_t*)(wa[nt] + up + k + 32 * u);
+                }
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                w0[nt] = *(const moe_bf16x8_t*)(wa[nt] + k);
-                if (GATED) w1[nt] = *(const moe_bf16x8_t*)(wa[nt] + up + k);
+                for (int mt = 0; mt < MT; ++mt) x[u][mt] = *(const moe_bf16x8_t*)(xp[mt] + k + 32 * u);
             }
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) x[mt] = *(const moe_bf16x8_t*)(xp[mt] + k);
+            for (int u = 0; u < KU; ++u)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        a[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u][nt], x[u][mt], a[nt][mt], 0, 0, 0);
+                        if (GATED)
+                            g[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u][nt], x[u][mt], g[nt][mt], 0, 0, 0);
+                    }
         }
-        if (AHEAD) {
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                w0n[nt] = *(const moe_bf16x8_t*)(wa[nt] + kn);
-                if (GATED) w1n[nt] = *(const moe_bf16x8_t*)(wa[nt] + up + kn);
-            }
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) xn[mt] = *(const moe_bf16x8_t*)(xp[mt] + kn);
+    } else {
+        // the operands of the next 32 k are asked for before this step's products are issued
+        moe_bf16x8_t w0[NT], w1[NT], x[MT];
+    #pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            w0[nt] = *(const moe_bf16x8_t*)(wa[nt]);
+            if (GATED) w1[nt] = *(const moe_bf16x8_t*)(wa[nt] + up);
         }
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                a[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[nt], x[mt], a[nt][mt], 0, 0, 0);
-                if (GATED)
-                    g[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[nt], x[mt], g[nt][mt], 0, 0, 0);
+    #pragma unroll
+        for (int mt = 0; mt < MT; ++mt) x[mt] = *(const moe_bf16x8_t*)(xp[mt]);
+        for (int k = 0; k < K; k += 32) {
+            moe_bf16x8_t w0n[NT], w1n[NT], xn[MT];
+            const int kn = k + 32 < K ? k + 32 : k;            // the last step loads its own again
+            if (!AHEAD && k > 0) {
+                // (many accumulators: no second set of operands; other waves hide the loads)
+    #pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    w0[nt] = *(const moe_bf16x8_t*)(wa[nt] + k);
+                    if (GATED) w1[nt] = *(const moe_bf16x8_t*)(wa[nt] + up + k);
+                }
+    #pragma unroll
+                for (int mt = 0; mt < MT; ++mt) x[mt] = *(const moe_bf16x8_t*)(xp[mt] + k);
             }
-        if (AHEAD) {
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                w0[nt] = w0n[nt];
-                if (GATED) w1[nt] = w1n[nt];
+            if (AHEAD) {
+    #pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    w0n[nt] = *(const moe_bf16x8_t*)(wa[nt] + kn);
+                    if (GATED) w1n[nt] = *(const moe_bf16x8_t*)(wa[nt] + up + kn);
+                }
+    #pragma unroll
+                for (int mt = 0; mt < MT; ++mt) xn[mt] = *(const moe_bf16x8_t*)(xp[mt] + kn);
             }
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) x[mt] = xn[mt];
+    #pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+    #pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    a[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[nt], x[mt], a[nt][mt], 0, 0, 0);
+                    if (GATED)
+                        g[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[nt], x[mt], g[nt][mt], 0, 0, 0);
+                }
+            if (AHEAD) {
+    #pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    w0[nt] = w0n[nt];
+                    if (GATED) w1[nt] = w1n[nt];
+                }
+    #pragma unroll
+                for (int mt = 0; mt < MT; ++mt) x[mt] = xn[mt];
+            }
         }
     }
     // a[nt][mt][i] belongs to the pair of row mt * 16 + r and column n0 + 16 nt + 4 q + i
@@ -432,20 +488,24 @@ extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int g
         return ILLM_ERR_ARG;
     if (max_tiles == 0) return ILLM_OK;
     hipStream_t st = (hipStream_t)stream;
-#define GO(MT_, NT_, G_)                                                                           \
+#define GO(MT_, NT_, G_, KU_)                                                                      \
     do {                                                                                           \
         const dim3 grid(max_tiles, (N + 64 * NT_ - 1) / (64 * NT_));                               \
         if (grid.y > 65535) return ILLM_ERR_ARG;                                                   \
-        hipLaunchKernelGGL((moe_rows_mfma_kernel<MT_, NT_, G_, (MT_ * NT_ <= 16)>), grid, dim3(256), 0, st, \
+        hipLaunchKernelGGL((moe_rows_mfma_kernel<MT_, NT_, G_, (MT_ * NT_ <= 16), KU_>), grid, dim3(256), 0, st, \
                            (const bf16_t*)X, x_div, (const bf16_t*)W, order, tiles, max_tiles,     \
                            (bf16_t*)Y, N, K);                                                      \
     } while (0)
     if (tile_rows == 16 && (long)max_tiles * ((N + 255) / 256) < 512) {
         // few tiles (single tokens): 16 columns a wave, so that more waves share the reading
-        if (gated) GO(1, 1, true); else GO(1, 1, false);
-    } else if (tile_rows == 16) { if (gated) GO(1, 4, true); else GO(1, 4, false); }
-    else if (tile_rows == 32) { if (gated) GO(2, 4, true); else GO(2, 4, false); }
-    else { if (gated) GO(4, 2, true); else GO(4, 4, false); }    // wider column blocks measured slower
+        if (K % 256 == 0) { if (gated) GO(1, 1, true, 8); else GO(1, 1, false, 8); }
+        else { if (gated) GO(1, 1, true, 1); else GO(1, 1, false, 1); }
+    } else if (tile_rows == 16) {
+        if (K % 64 == 0) { if (gated) GO(1, 4, true, 2); else GO(1, 4, false, 2); }
+        else { if (gated) GO(1, 4, true, 1); else GO(1, 4, false, 1); }
+    }
+    else if (tile_rows == 32) { if (gated) GO(2, 4, true, 1); else GO(2, 4, false, 1); }
+    else { if (gated) GO(4, 2, true, 1); else GO(4, 4, false, 1); }    // wider column blocks measured slower
 #undef GO
     return illm_launch_status();
 }

@@ -1143,7 +1143,7 @@ def latent_attn_decode(y: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor, 
                      device=y.device)
     _check(_lib().illm_latent_absorb_q(_p(y), _code(y), y.shape[1], _p(w_uk), _code(w_uk), _p(qa),
                                        _code(qa), B, H, dn, dr, R, _stream()), "latent_absorb_q")
-    partial = torch.empty((B, H, nsplit, R + 2), dtype=torch.float32, device=y.device)
+    partial = torch.empty((B, H, nsplit, R + 4), dtype=torch.float32, device=y.device)
     if cache_t is not None:
         _need(latent_decode_mfma_fits(cache, cache_t, R, dr, page_size) and
               cache_t.shape == (cache.shape[0], R, page_size, 1) and cache_t.is_contiguous(),
