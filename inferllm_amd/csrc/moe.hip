@@ -480,6 +480,124 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __re
     }
 }
 
+// Tiles of 64 pairs (prompts), K % 64 == 0: as above with the tile's X rows shared by the block's
+// four waves through LDS, 64 k at a time in two buffers (a thread brings 32 bytes of one row; the
+// 16-byte pieces of a row are placed at piece ^ (row % 8), so that the 16 rows a product's operand
+// reads lie in different banks); one barrier a slab.  W stays a stream of each wave's own rows,
+// asked for one slab ahead.
+template <int NT, bool GATED>
+__global__ void __launch_bounds__(256)
+moe_rows_mfma_lds_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __restrict__ W,
+                         const int32_t* __restrict__ order, const int32_t* __restrict__ tiles,
+                         int max_tiles, bf16_t* __restrict__ Y, int N, int K) {
+    constexpr int MT = 4;
+    __shared__ uint4 xs[2][64 * 8];
+    const int tile = blockIdx.x;
+    if (tile >= tiles[3 * (size_t)max_tiles]) return;          // the whole block leaves together
+    const int e = tiles[3 * (size_t)tile], first = tiles[3 * (size_t)tile + 1];
+    const int n = tiles[3 * (size_t)tile + 2];
+    const int w = wave_index(), lane = threadIdx.x & 63;
+    const int r = lane & 15, q = lane >> 4;
+    const int lr = threadIdx.x >> 2, lc = (threadIdx.x & 3) * 2;       // the row and pieces this thread brings
+    const bf16_t* lx = X + (size_t)(order[first + (lr < n ? lr : n - 1)] / x_div) * K + lc * 8;
+    const int s0 = lr * 8 + (lc ^ (lr & 7)), s1 = lr * 8 + ((lc + 1) ^ (lr & 7));
+    int pair[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int i = mt * 16 + r;
+        pair[mt] = order[first + (i < n ? i : n - 1)];
+    }
+    const size_t wrows = GATED ? 2 * (size_t)N : (size_t)N;
+    const int n0 = (blockIdx.y * 4 + w) * 16 * NT;             // (a wave beyond N works on row N - 1 and writes nothing)
+    const bf16_t* wa[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int wr = n0 + nt * 16 + r < N ? n0 + nt * 16 + r : N - 1;
+        wa[nt] = W + ((size_t)e * wrows + wr) * K + q * 8;
+    }
+    const size_t up = (size_t)N * K;
+    moe_f32x4_t a[NT][MT], g[NT][MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            a[nt][mt] = (moe_f32x4_t){0.f, 0.f, 0.f, 0.f};
+            g[nt][mt] = a[nt][mt];
+        }
+    moe_bf16x8_t w0[2][NT], w1[2][NT];
+    uint4 xa = *(const uint4*)lx, xb = *(const uint4*)(lx + 8);
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            w0[u][nt] = *(const moe_bf16x8_t*)(wa[nt] + 32 * u);
+            if (GATED) w1[u][nt] = *(const moe_bf16x8_t*)(wa[nt] + up + 32 * u);
+        }
+    xs[0][s0] = xa;
+    xs[0][s1] = xb;
+    __syncthreads();
+    for (int k = 0; k < K; k += 64) {
+        const int buf = (k >> 6) & 1;
+        const int kn = k + 64 < K ? k + 64 : k;                  // the last slab asks for itself again
+        moe_bf16x8_t w0n[2][NT], w1n[2][NT];
+        xa = *(const uint4*)(lx + kn);
+        xb = *(const uint4*)(lx + kn + 8);
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                w0n[u][nt] = *(const moe_bf16x8_t*)(wa[nt] + kn + 32 * u);
+                if (GATED) w1n[u][nt] = *(const moe_bf16x8_t*)(wa[nt] + up + kn + 32 * u);
+            }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            moe_bf16x8_t x[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const uint4 v = xs[buf][(mt * 16 + r) * 8 + ((u * 4 + q) ^ (r & 7))];
+                x[mt] = *(const moe_bf16x8_t*)&v;
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    a[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u][nt], x[mt], a[nt][mt], 0, 0, 0);
+                    if (GATED)
+                        g[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u][nt], x[mt], g[nt][mt], 0, 0, 0);
+                }
+        }
+        xs[buf ^ 1][s0] = xa;
+        xs[buf ^ 1][s1] = xb;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                w0[u][nt] = w0n[u][nt];
+                if (GATED) w1[u][nt] = w1n[u][nt];
+            }
+        __syncthreads();
+    }
+    if (n0 >= N) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        if (mt * 16 + r >= n) continue;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int col = n0 + 16 * nt + 4 * q + i;
+                if (col >= N) continue;
+                float v = a[nt][mt][i];
+                if (GATED) {
+                    const float gate = bf16_to_f32(f32_to_bf16(a[nt][mt][i]));
+                    const float upv = bf16_to_f32(f32_to_bf16(g[nt][mt][i]));
+                    v = (gate / (1.0f + expf(-gate))) * upv;
+                }
+                Y[(size_t)pair[mt] * N + col] = f32_to_bf16(v);
+            }
+    }
+}
+
 extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int gated, int tile_rows,
                                   const int32_t* order, const int32_t* tiles, int max_tiles,
                                   void* Y, int N, int K, void* stream) {
@@ -488,6 +606,18 @@ extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int g
         return ILLM_ERR_ARG;
     if (max_tiles == 0) return ILLM_OK;
     hipStream_t st = (hipStream_t)stream;
+    if (tile_rows == 64 && K % 64 == 0) {
+        const int nt = gated ? 2 : 4;
+        const dim3 grid(max_tiles, (N + 64 * nt - 1) / (64 * nt));
+        if (grid.y > 65535) return ILLM_ERR_ARG;
+        if (gated)
+            hipLaunchKernelGGL((moe_rows_mfma_lds_kernel<2, true>), grid, dim3(256), 0, st, (const bf16_t*)X,
+                               x_div, (const bf16_t*)W, order, tiles, max_tiles, (bf16_t*)Y, N, K);
+        else
+            hipLaunchKernelGGL((moe_rows_mfma_lds_kernel<4, false>), grid, dim3(256), 0, st, (const bf16_t*)X,
+                               x_div, (const bf16_t*)W, order, tiles, max_tiles, (bf16_t*)Y, N, K);
+        return illm_launch_status();
+    }
 #define GO(MT_, NT_, G_, KU_)                                                                      \
     do {                                                                                           \
         const dim3 grid(max_tiles, (N + 64 * NT_ - 1) / (64 * NT_));                               \
