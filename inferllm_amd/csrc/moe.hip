@@ -629,6 +629,8 @@ extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int g
     if (tile_rows == 16 && (long)max_tiles * ((N + 255) / 256) < 512) {
         // few tiles (single tokens): 16 columns a wave, so that more waves share the reading
         if (K % 256 == 0) { if (gated) GO(1, 1, true, 8); else GO(1, 1, false, 8); }
+        else if (K % 128 == 0) { if (gated) GO(1, 1, true, 4); else GO(1, 1, false, 4); }
+        else if (K % 64 == 0) { if (gated) GO(1, 1, true, 2); else GO(1, 1, false, 2); }
         else { if (gated) GO(1, 1, true, 1); else GO(1, 1, false, 1); }
     } else if (tile_rows == 16) {
         if (K % 64 == 0) { if (gated) GO(1, 4, true, 2); else GO(1, 4, false, 2); }
