@@ -39,8 +39,8 @@ MIXED = {"architecture": "Rabapel", "vocab": 300, "width": 96, "norm": {"eps": 1
              {"type": "latent_attention", "mixer": _mixer(5, 8, 16, 40, 64, 0.2, dims=12, base=5000.0),
               "mlp": _moe(48, 5, 3, identity=2, shared=72)},
              {"type": "latent_attention", "mixer": _mixer(16, 4, 4, 6, 130, 0.5, window=33), "mlp": None},
-             {"type": "latent_attention", "mixer": _mixer(2, 32, 32, 20, 24, 0.11, base=250000.0,
-                                                           scaling={"factor": 8.0, "original": 128, "fast": 32.0, "slow": 1.0}),
+             {"type": "latent_attention", "mixer": _mixer(2, 32, 32, 20, 24, 0.11, base=300000.0,
+                                                           scaling={"factor": 5.0, "original": 96, "fast": 20.0, "slow": 1.5}),
               "mlp": _moe(40, 3, 1)},
          ]}
 
@@ -57,7 +57,7 @@ ODD = {"architecture": "Rabapel", "vocab": 131, "width": 90, "norm": {"eps": 3e-
 # one layer, for tests that plant a key (`plant_key`)
 def single(window=None, heads=4, dim=16, rot_dim=8, vdim=12, rank=48, mlp=None, width=64, vocab=200):
     return {"architecture": "Rabapel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
-            "embedding": {"scale": 0.5},
+            "embedding": {"scale": 0.6},
             "layers": [{"type": "latent_attention",
                         "mixer": _mixer(heads, dim, rot_dim, vdim, rank, 0.25, window=window, scaling=YARN),
                         "mlp": mlp}]}

@@ -50,7 +50,7 @@ def test_config_errors_name_the_key(change):
 
 @pytest.mark.parametrize("rot", [
     {"base": 10000.0, "dims": 8, "scaling": YARN},
-    {"base": 250000.0, "dims": 32, "scaling": {"factor": 8.0, "original": 512, "fast": 32.0, "slow": 1.0}},
+    {"base": 300000.0, "dims": 24, "scaling": {"factor": 5.0, "original": 256, "fast": 20.0, "slow": 1.5}},
     {"base": 5000.0, "dims": 12},
     {"base": 100.0, "dims": 4, "scaling": {"factor": 2.0, "original": 16, "fast": 1.0, "slow": 1.0}},
 ])
