@@ -299,7 +299,9 @@ def test_router_kernel(n_out, top):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("E,F,n_real,n_id,top,T", [(64, 40, 5, 2, 3, 37), (90, 30, 2, 0, 1, 9),
-                                                   (128, 96, 12, 4, 2, 300)])
+                                                   (128, 96, 12, 4, 2, 300), (96, 64, 6, 1, 2, 3),
+                                                   (160, 32, 4, 0, 3, 40), (256, 128, 3, 1, 2, 700),
+                                                   (320, 64, 12, 4, 2, 1000), (512, 160, 5, 0, 1, 1)])
 def test_expert_kernels(dtype, E, F, n_real, n_id, top, T):
     """Grouping, the experts' products and the weighted sum against a loop over tokens."""
     from inferllm_amd.kernels import ops
