@@ -90,6 +90,31 @@ def test_long_decoding_past_windows_and_pages(tmp_path_factory, dtype):
     eng.free_slot(s)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads,dim,rot_dim,vdim,rank,window", [(20, 64, 32, 96, 256, 70), (3, 160, 64, 224, 208, None),
+                                                                (33, 16, 16, 24, 512, 129)])
+def test_wide_heads_and_long_latents(tmp_path_factory, heads, dim, rot_dim, vdim, rank, window, dtype):
+    """Heads of up to 224 dims, latents of 208 to 512, 3 to 33 heads (the kernels' other branches:
+    more accumulators, several groups of heads, generic prompt attention)."""
+    from inferllm_amd import StepEntry
+    config = single(window=window, heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, rank=rank,
+                    mlp={"kind": "dense", "ff": 96}, width=128)
+    d = write_model(tmp_path_factory.getbasetemp(), config, seed=heads, dtype=STORE[dtype], gain=2.0)
+    w = weights64(d)
+    eng = engine_for(d, dtype)
+    reqs = [random_ids(n, config["vocab"], n) for n in (170, 66)]
+    slots = [eng.alloc_slot() for _ in reqs]
+    cut = [len(r) - 12 for r in reqs]
+    out = eng.step([StepEntry(s, r[:k], list(range(k))) for s, r, k in zip(slots, reqs, cut)])
+    got = [[out[:cut[0]].clone()], [out[cut[0]:].clone()]]
+    for t in range(12):
+        o = eng.step([StepEntry(slots[i], [reqs[i][cut[i] + t]], [0]) for i in range(2)])
+        for i in range(2):
+            got[i].append(o[i:i + 1].clone())
+    for i, r in enumerate(reqs):
+        close(torch.cat(got[i]), P.forward(config, w, r), dtype, f"request {i}")
+
+
 @pytest.mark.parametrize("graphs", [True, False])
 def test_portions_of_a_prompt(tmp_path_factory, graphs):
     """A prompt fed in portions of 2 to 90 tokens (and single ones between) gives what the whole
