@@ -35,6 +35,12 @@ int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, int planes, size
                      const void* w, int w_dt, void* out, int out_dt, const int32_t* row_idx,
                      int rows, int E, float eps, void* stream);
 
+// The same with a second addend of delta's shape (may be null): v = x + (delta + delta2), the two
+// outputs of a block whose parts read the same rows.
+int illm_add2_rmsnorm(float* x, const void* delta, int delta_dt, int planes, size_t plane_stride,
+                      const void* delta2, int delta2_dt, const void* w, int w_dt, void* out,
+                      int out_dt, const int32_t* row_idx, int rows, int E, float eps, void* stream);
+
 // out[t, f] = silu(gate_up[t, f]) * gate_up[t, F + f].
 int illm_silu_mul(const void* gate_up, void* out, int dt, int T, int F, void* stream);
 

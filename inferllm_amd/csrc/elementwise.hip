@@ -83,6 +83,7 @@ __device__ __forceinline__ float ld_planes(const void* delta, int dt, size_t i, 
 
 __global__ void add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ delta,
                                    int delta_dt, int planes, size_t plane_stride,
+                                   const void* __restrict__ delta2, int delta2_dt,
                                    const void* __restrict__ w, int w_dt,
                                    void* __restrict__ out, int out_dt,
                                    const int32_t* __restrict__ row_idx, int E, float eps) {
@@ -94,7 +95,9 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict
     for (int i = threadIdx.x; i < E; i += blockDim.x) {
         float v = x[ib + i];
         if (delta) {
-            v += ld_planes(delta, delta_dt, ib + i, planes, plane_stride);
+            float d = ld_planes(delta, delta_dt, ib + i, planes, plane_stride);
+            if (delta2) d += ld_f(delta2, delta2_dt, ib + i);
+            v += d;
             if (!row_idx) x[ib + i] = v;
         }
         ss += v * v;
@@ -103,7 +106,11 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict
     const float scale = 1.0f / sqrtf(ss / (float)E + eps);
     for (int i = threadIdx.x; i < E; i += blockDim.x) {
         float v = x[ib + i];
-        if (delta && row_idx) v += ld_planes(delta, delta_dt, ib + i, planes, plane_stride);
+        if (delta && row_idx) {
+            float d = ld_planes(delta, delta_dt, ib + i, planes, plane_stride);
+            if (delta2) d += ld_f(delta2, delta2_dt, ib + i);
+            v += d;
+        }
         st_f(out, out_dt, ob + i, (v * scale) * ld_f(w, w_dt, i));
     }
 }
@@ -134,7 +141,8 @@ __device__ __forceinline__ void st4_f(void* p, int dt, size_t i4, float4 v) {
 template <int NV, int TH>
 __global__ void __launch_bounds__(TH)
 add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, int delta_dt,
-                       int planes, size_t plane_stride4,
+                       int planes, size_t plane_stride4, const void* __restrict__ delta2,
+                       int delta2_dt,
                        const void* __restrict__ w, int w_dt, void* __restrict__ out, int out_dt,
                        const int32_t* __restrict__ row_idx, int E, float eps) {
     __shared__ float red[16];
@@ -172,6 +180,10 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, in
                         d.x += e[t].x; d.y += e[t].y; d.z += e[t].z; d.w += e[t].w;
                     }
                 }
+                if (delta2) {                         // a second addend: (delta + delta2) first
+                    const float4 e2 = ld4_f(delta2, delta2_dt, ib + i);
+                    d.x += e2.x; d.y += e2.y; d.z += e2.z; d.w += e2.w;
+                }
                 v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
                 if (!row_idx) ((float4*)x)[ib + i] = v[j];
             }
@@ -193,10 +205,11 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, in
     }
 }
 
-extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, int planes,
-                                size_t plane_stride, const void* w, int w_dt, void* out,
-                                int out_dt, const int32_t* row_idx, int rows, int E, float eps,
-                                void* stream) {
+extern "C" int illm_add2_rmsnorm(float* x, const void* delta, int delta_dt, int planes,
+                                 size_t plane_stride, const void* delta2, int delta2_dt,
+                                 const void* w, int w_dt, void* out, int out_dt,
+                                 const int32_t* row_idx, int rows, int E, float eps, void* stream) {
+    if (delta2 && (!delta || !illm_dtype_ok(delta2_dt))) return ILLM_ERR_ARG;
     if (rows < 0 || E <= 0 || !illm_dtype_ok(w_dt) || !illm_dtype_ok(out_dt) ||
         (delta && (!illm_dtype_ok(delta_dt) || planes < 1 ||
                    (planes > 1 && E % 4 == 0 && plane_stride % 4))))
@@ -205,8 +218,8 @@ extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, int p
     hipStream_t st = (hipStream_t)stream;
 #define VEC(NV_, TH_)                                                                         \
     hipLaunchKernelGGL((add_rmsnorm_vec_kernel<NV_, TH_>), dim3(rows), dim3(TH_), 0, st, x,   \
-                       delta, delta_dt, planes, plane_stride / 4, w, w_dt, out, out_dt, row_idx, \
-                       E, eps)
+                       delta, delta_dt, planes, plane_stride / 4, delta2, delta2_dt, w, w_dt, out,  \
+                       out_dt, row_idx, E, eps)
     // few rows (decoding): wide blocks, one group of 4 floats per thread, to shorten the row's
     // critical path; many rows: narrow blocks so that more rows are in flight per CU
     if (E % 4 == 0 && rows <= 128 && E > 1024 && E <= 4096) VEC(1, 1024);
@@ -217,9 +230,18 @@ extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, int p
     else if (E % 4 == 0 && E <= 8192) VEC(8, 256);
     else
         hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(rows), dim3(256), 0, st, x, delta, delta_dt,
-                           planes, plane_stride, w, w_dt, out, out_dt, row_idx, E, eps);
+                           planes, plane_stride, delta2, delta2_dt, w, w_dt, out, out_dt, row_idx, E,
+                           eps);
 #undef VEC
     return illm_launch_status();
+}
+
+extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, int planes,
+                                size_t plane_stride, const void* w, int w_dt, void* out,
+                                int out_dt, const int32_t* row_idx, int rows, int E, float eps,
+                                void* stream) {
+    return illm_add2_rmsnorm(x, delta, delta_dt, planes, plane_stride, nullptr, 0, w, w_dt, out,
+                             out_dt, row_idx, rows, E, eps, stream);
 }
 
 // ---------------------------------------------------------------- silu * up

@@ -134,8 +134,14 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
 
     Without `row_idx` the sum is written back to `x`.  With `row_idx` only those
     rows are normed (and `x` is left as it is).  `delta` may be [S, T, E]: the planes of a
-    product whose K was split (`linear_planes`), added in order.
+    product whose K was split (`linear_planes`), added in order; or a pair of tensors of x's shape
+    (the outputs of two parts that read the same rows): x + (first + second).
     """
+    delta2 = None
+    if isinstance(delta, (tuple, list)):
+        delta, delta2 = delta
+        _need(delta.shape == x.shape and delta2.shape == x.shape, "add_rmsnorm: a pair needs x's shape")
+        _gpu(delta2)
     _gpu(x, delta, weight, row_idx)
     _i32(row_idx)
     _need(x.dtype == torch.float32 and x.dim() == 2, "add_rmsnorm: x must be float32 [T, E]")
@@ -149,9 +155,10 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         _need(delta.shape[-2:] == x.shape, "add_rmsnorm: delta must have x's shape")
     rows = T if row_idx is None else row_idx.numel()
     out = torch.empty((rows, E), dtype=out_dtype, device=x.device)
-    _check(_lib().illm_add_rmsnorm(
+    _check(_lib().illm_add2_rmsnorm(
         _p(x), _p(delta), _code(delta) if delta is not None else 0, planes,
-        ctypes.c_size_t(T * E), _p(weight), _code(weight),
+        ctypes.c_size_t(T * E), _p(delta2), _code(delta2) if delta2 is not None else 0,
+        _p(weight), _code(weight),
         _p(out), _code(out), _p(row_idx), rows, E, ctypes.c_float(eps), _stream()), "add_rmsnorm")
     return out
 

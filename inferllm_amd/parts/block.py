@@ -50,17 +50,27 @@ class PreNormBlock(Block):
 class ParallelBlock(Block):
     """x <- x + (mixer(h) + feed_forward(h)) with h = norm(x): one norm, both parts read its rows.
 
-    The two outputs are added in float32 and the sum is what the block leaves for the next norm
-    to add to the stream.  A feed-forward that returns None (a layer without one) leaves the
-    mixer's output alone.
+    The two outputs are left for the next norm to add to the stream as (mixer + feed-forward) in
+    float32: as a pair, if that norm says it adds pairs in its own kernel (`Norm.adds_pairs`), else
+    as their float32 sum (`ops.sum_rows`).  A feed-forward that returns None (a layer without one)
+    leaves the mixer's output alone.
     """
 
     graph_safe_prompts = True
 
-    def forward(self, x, pending, ctx: StepContext, line, writes_cache):
+    takes_next_norm = True           # to know whether the norm that follows adds a pair itself
+    takes_prepared_rows = True       # (prepared rows mean: the sum is in x already)
+
+    def forward(self, x, pending, ctx: StepContext, line, writes_cache, next_norm=None):
         if isinstance(pending, ops.NormedRows):
             pending = None                       # its sum is in x already
+        if isinstance(pending, tuple) and not getattr(self.mixer_norm, "adds_pairs", False):
+            pending = ops.sum_rows(*pending)
         h = self.mixer_norm.forward(x, pending, ctx)
         a = self.mixer.forward(h, ctx, line, writes_cache, self.position)
         f = self.feed_forward.forward(h, ctx)
-        return a if f is None else ops.sum_rows(a, f)
+        if f is None:
+            return a
+        if next_norm is not None and getattr(next_norm, "adds_pairs", False):
+            return (a, f)
+        return ops.sum_rows(a, f)

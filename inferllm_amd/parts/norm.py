@@ -21,6 +21,9 @@ class RMSNorm(Norm):
     graph_safe_prompts = True
 
     adds_planes = True
+    # `forward` also takes `delta` as a pair of tensors (two parts' outputs for the same rows),
+    # added as x + (first + second) in the norm's own kernel
+    adds_pairs = True
 
     def __init__(self, size: int, eps: float, tensors=None):
         super().__init__(tensors)

@@ -20,6 +20,8 @@ def embed(tokens, table, scale=1.0):
 
 
 def add_rmsnorm(x, delta, weight, eps, out_dtype, row_idx=None):
+    if isinstance(delta, (tuple, list)):               # two parts' outputs for the same rows
+        delta = delta[0].to(F64) + delta[1].to(F64)
     if delta is not None:
         if delta.dim() == 3:                           # planes of a split product
             delta = delta.to(F64).sum(0)

@@ -309,6 +309,26 @@ def test_architecture_is_chosen_by_config_and_refuses_what_it_lacks(tmp_path_fac
 
 
 # ---------------------------------------------------------------- mechanisms alone
+@pytest.mark.parametrize("E", [96, 90, 2048])
+def test_norm_adds_a_pair_of_outputs(E):
+    """x + (a + b) and the norm in one kernel, for all rows and for picked rows."""
+    from inferllm_amd.kernels import ops
+    import kernel_refs as K
+    g = torch.Generator().manual_seed(E)
+    x = torch.randn((7, E), generator=g)
+    a = torch.randn((7, E), generator=g).to(torch.bfloat16)
+    b = torch.randn((7, E), generator=g)
+    wt = torch.rand((E,), generator=g) + 0.5
+    for rows in (None, torch.tensor([5, 0, 2], dtype=torch.int32)):
+        xg, xr = x.clone().cuda(), x.clone()
+        got = ops.add_rmsnorm(xg, (a.cuda(), b.cuda()), wt.cuda(), 1e-5, torch.float32,
+                              rows.cuda() if rows is not None else None)
+        want = K.add_rmsnorm(xr, (a, b), wt, 1e-5, torch.float32, rows)
+        assert float((got.cpu() - want).abs().max()) < 1e-5
+        assert float((xg.cpu() - xr).abs().max()) < 1e-6
+
+
+
 @pytest.mark.parametrize("n_out,top", [(7, 3), (16, 2), (130, 8), (3, 1)])
 def test_router_kernel(n_out, top):
     from inferllm_amd.kernels import ops
