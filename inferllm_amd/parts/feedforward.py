@@ -69,7 +69,7 @@ class NoFeedForward(FeedForward):
         return None
 
 
-_ACTIVATIONS = {"relu_squared": ops.relu_squared}
+_ACTIVATIONS = {"relu_squared": "relu_squared"}        # activation -> the op that computes it
 
 
 @register_part("feed_forward", "dense_activation")
@@ -97,7 +97,8 @@ class DenseActivation(FeedForward):
         return (("plain", self.w_down, {}),)
 
     def forward(self, h, ctx: StepContext):
-        return ops.linear(_ACTIVATIONS[self.activation](ops.linear(h, self.w_up)), self.w_down)
+        act = getattr(ops, _ACTIVATIONS[self.activation])
+        return ops.linear(act(ops.linear(h, self.w_up)), self.w_down)
 
 
 @register_part("feed_forward", "routed_experts")

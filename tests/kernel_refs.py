@@ -249,10 +249,140 @@ def sample(logits, temperature, top_k, top_p, repeat_penalty, last_tokens, seeds
     return torch.tensor(out, dtype=torch.int32)
 
 
+
+# ---------------------------------------------------------------- latent attention
+def sum_rows(a, b):
+    return (a.to(F64) + b.to(F64)).to(torch.float32)
+
+
+def relu_squared(x):
+    return (torch.relu(x.to(F64)) ** 2).to(x.dtype)
+
+
+def _rotate_pairs(v, cc, ss, rot):
+    """Pairs (2i, 2i+1), i < rot/2, of the last axis of v (float64, changed in place)."""
+    a, b = v[..., 0:rot:2].clone(), v[..., 1:rot:2].clone()
+    v[..., 0:rot:2] = a * cc - b * ss
+    v[..., 1:rot:2] = b * cc + a * ss
+
+
+def latent_rope_store(y, H, dn, dr, R, rot, cos_sin, norm_w, eps, row_pos, row_slot, slot_len,
+                      cache, page_table, page_size, ring, want_rows, cache_t=None):
+    T, q_cols = y.shape[0], H * (dn + dr)
+    down = y[:, q_cols:q_cols + R + dr].to(F64)
+    c = down[:, :R]
+    c = c / torch.sqrt((c * c).mean(dim=-1, keepdim=True) + eps) * norm_w.to(F64)
+    kr = down[:, R:].clone()
+    if cos_sin is not None:
+        cs = cos_sin[row_pos.long()].to(F64)                      # [T, rot/2, 2]
+        _rotate_pairs(kr, cs[..., 0], cs[..., 1], rot)
+        q = y[:, :q_cols].to(F64).reshape(T, H, dn + dr)
+        tail = q[:, :, dn:].clone()
+        _rotate_pairs(tail, cs[:, None, :, 0], cs[:, None, :, 1], rot)
+        q[:, :, dn:] = tail
+        y[:, :q_cols] = q.reshape(T, q_cols).to(y.dtype)
+    c, kr = c.to(y.dtype), kr.to(y.dtype)
+    if cache is not None:
+        for t in range(T):
+            slot, pos = int(row_slot[t]), int(row_pos[t])
+            if ring > 0 and slot_len is not None:
+                if pos // page_size + ring <= (int(slot_len[slot]) - 1) // page_size:
+                    continue
+            page, r = cache_offsets(page_table, slot, pos, page_size, ring)
+            cache[page, r, :R] = c[t]
+            cache[page, r, R:] = kr[t]
+            if cache_t is not None:
+                cache_t[page, :, r, 0] = c[t]
+    return (c, kr) if want_rows else (None, None)
+
+
+def latent_pack(y, kvu, kr, H, dn, dr, dv, P):
+    T = y.shape[0]
+    out = torch.zeros((T, 3, H, P), dtype=y.dtype)
+    out[:, 0, :, :dn + dr] = y[:, :H * (dn + dr)].reshape(T, H, dn + dr)
+    out[:, 1, :, :dn] = kvu[:, :H * dn].reshape(T, H, dn)
+    out[:, 1, :, dn:dn + dr] = kr[:, None, :]
+    out[:, 2, :, :dv] = kvu[:, H * dn:].reshape(T, H, dv)
+    return out.reshape(T, 3 * H * P)
+
+
+def latent_gate(attn, y, gate_off, H, dv, P):
+    T = y.shape[0]
+    g = torch.sigmoid(y[:, gate_off:gate_off + H].to(F64))
+    return (attn.to(F64).reshape(T, H, P)[:, :, :dv] * g[:, :, None]).reshape(T, H * dv).to(y.dtype)
+
+
+def latent_decode_splits(B, H, longest, mfma=False):
+    return 1
+
+
+def latent_decode_mfma_fits(cache, cache_t, R, dr, page_size):
+    return False
+
+
+def latent_attn_decode(y, w_uk, w_uv, gate_off, cache, page_table, page_size, ring, seq_slot, seq_len,
+                       len_more, H, dn, dr, R, dv, scale, window, nsplit, cache_t=None):
+    B = y.shape[0]
+    out = torch.zeros((B, H * dv), dtype=y.dtype)
+    wk, wv = w_uk.to(F64).reshape(H, dn, R), w_uv.to(F64).reshape(H, dv, R)
+    for b in range(B):
+        slot, L = int(seq_slot[b]), int(seq_len[b]) + len_more
+        lo = max(0, L - window) if window and window > 0 else 0
+        rows = torch.stack([cache[cache_offsets(page_table, slot, p, page_size, ring)] for p in range(lo, L)]).to(F64)
+        q = y[b, :H * (dn + dr)].to(F64).reshape(H, dn + dr)
+        gate = torch.sigmoid(y[b, gate_off:gate_off + H].to(F64))
+        for h in range(H):
+            qa = torch.cat([q[h, :dn] @ wk[h], q[h, dn:]])
+            p = torch.softmax((rows @ qa) * scale, dim=0)
+            out[b, h * dv:(h + 1) * dv] = ((wv[h] @ (p @ rows[:, :R])) * gate[h]).to(y.dtype)
+    return out
+
+
+# ---------------------------------------------------------------- routed feed-forward
+def few_outputs_f32(x, w):
+    return (x.to(F64) @ w.to(F64).t()).to(torch.float32)
+
+
+def moe_route(z, correction, top):
+    s = torch.softmax(z.to(F64), dim=-1)
+    pick = s + correction.to(F64) if correction is not None else s
+    idx = torch.topk(pick, top, dim=-1).indices
+    return idx.to(torch.int32), torch.gather(s, 1, idx).to(torch.float32)
+
+
+def moe_experts(h, idx, w_gate_up, w_down):
+    T, top = idx.shape
+    F = w_gate_up.shape[1] // 2
+    y = torch.zeros((T * top, h.shape[1]), dtype=h.dtype)
+    for t in range(T):
+        for k in range(top):
+            e = int(idx[t, k])
+            if e < w_gate_up.shape[0]:
+                gu = w_gate_up[e].to(F64) @ h[t].to(F64)
+                y[t * top + k] = (w_down[e].to(F64) @ (torch.nn.functional.silu(gu[:F]) * gu[F:])).to(h.dtype)
+    return y
+
+
+def moe_combine(h, idx, wt, y, n_real, shared=None, shared_gate=None):
+    T, top = idx.shape
+    out = torch.zeros(h.shape, dtype=F64)
+    for t in range(T):
+        for k in range(top):
+            v = y[t * top + k] if int(idx[t, k]) < n_real else h[t]
+            out[t] += wt[t, k].to(F64) * v.to(F64)
+    if shared is not None:
+        g = torch.sigmoid(h.to(F64) @ shared_gate.to(F64))[:, None] if shared_gate is not None else 1.0
+        out = out + g * shared.to(F64)
+    return out.to(torch.float32)
+
+
 def patch(monkeypatch):
     """Put these functions in place of the GPU ops (CPU tests only)."""
     from inferllm_amd.kernels import ops
     for name in ("embed", "add_rmsnorm", "silu_mul", "rope_store", "linear", "gemm_generic", "gate_up_silu", "qkv_rope_store_fits",
                  "linear_add_fits",
-                 "attn_prefill", "attn_prefill_paged", "decode_splits", "attn_decode", "argmax", "sample"):
+                 "attn_prefill", "attn_prefill_paged", "decode_splits", "attn_decode", "argmax", "sample",
+                 "sum_rows", "relu_squared", "latent_rope_store", "latent_pack", "latent_gate",
+                 "latent_decode_splits", "latent_decode_mfma_fits", "latent_attn_decode",
+                 "few_outputs_f32", "moe_route", "moe_experts", "moe_combine"):
         monkeypatch.setattr(ops, name, globals()[name])

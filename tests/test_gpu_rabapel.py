@@ -309,6 +309,77 @@ def test_architecture_is_chosen_by_config_and_refuses_what_it_lacks(tmp_path_fac
 
 
 # ---------------------------------------------------------------- mechanisms alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,dn,dr,dv,R,rot,window", [(3, 16, 8, 24, 40, 8, 0), (16, 8, 16, 12, 64, 12, 70),
+                                                     (5, 24, 32, 40, 48, 32, 33), (20, 16, 16, 16, 128, 16, 0),
+                                                     (1, 0, 8, 8, 16, 8, 65)])
+def test_latent_kernels_alone(dtype, H, dn, dr, dv, R, rot, window):
+    """Norm, rotation and store of the latent rows, the packed rows for prompts, the gate, and
+    one token's attention over the paged latent cache (both kernels), against plain torch
+    (tests/kernel_refs.py), with scattered pages, a window's ring and unequal lengths."""
+    from inferllm_amd.kernels import ops
+    import kernel_refs as K
+    g = torch.Generator().manual_seed(H * 100 + R)
+    page, ring = 64, ((window + 62) // 64 + 1 if window else 0)
+    per_seq = ring or 4
+    lens = [130, 64, 200] if not window else [130, 64, 333]
+    table = torch.randperm(3 * per_seq, generator=g).to(torch.int32).view(3, per_seq)
+    ncols = H * (dn + dr) + R + dr + H
+    cos_sin = torch.randn((512, rot // 2, 2), generator=g)
+    norm_w = (torch.rand((R,), generator=g) + 0.5).to(dtype)
+    w_uk = (torch.randn((H * dn, R), generator=g) * 0.3).to(dtype)
+    w_uv = (torch.randn((H * dv, R), generator=g) * 0.3).to(dtype)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    transposed = dtype == torch.bfloat16 and R % 16 == 0 and (R + dr) % 8 == 0
+    cache_ref = torch.zeros((3 * per_seq + 1, page, R + dr), dtype=dtype)
+    cache_gpu = cache_ref.clone().cuda()
+    ct_ref = torch.zeros((3 * per_seq + 1, R, page, 1), dtype=dtype) if transposed else None
+    ct_gpu = ct_ref.clone().cuda() if transposed else None
+    # whole prompts: all rows of the three sequences in one call
+    T = sum(lens)
+    y = torch.randn((T, ncols), generator=g).to(dtype)
+    pos = torch.cat([torch.arange(n) for n in lens]).to(torch.int32)
+    slot = torch.cat([torch.full((n,), i) for i, n in enumerate(lens)]).to(torch.int32)
+    slot_len = torch.tensor(lens, dtype=torch.int32)
+    y_gpu = y.clone().cuda()
+    c_g, kr_g = ops.latent_rope_store(y_gpu, H, dn, dr, R, rot, cos_sin.cuda(), norm_w.cuda(), 1e-5, pos.cuda(),
+                                      slot.cuda(), slot_len.cuda(), cache_gpu, table.cuda(), page, ring, True, ct_gpu)
+    c_r, kr_r = K.latent_rope_store(y, H, dn, dr, R, rot, cos_sin, norm_w, 1e-5, pos, slot, slot_len, cache_ref,
+                                    table, page, ring, True, ct_ref)
+    for got, want in ((c_g, c_r), (kr_g, kr_r), (y_gpu, y), (cache_gpu, cache_ref)) + (((ct_gpu, ct_ref),) if transposed else ()):
+        assert float((got.double().cpu() - want.double()).abs().max()) <= tol * max(1.0, float(want.double().abs().max()))
+    cache_gpu.copy_(cache_ref)                      # the same bits on both sides from here on
+    if transposed:
+        ct_gpu.copy_(ct_ref)
+    kvu = torch.randn((T, H * (dn + dv)), generator=g).to(dtype)
+    P_ = -(-max(dn + dr, dv) // 16) * 16
+    packed = ops.latent_pack(y_gpu, kvu.cuda(), kr_g, H, dn, dr, dv, P_)
+    assert torch.equal(packed.cpu(), K.latent_pack(y_gpu.cpu(), kvu, kr_g.cpu(), H, dn, dr, dv, P_))
+    attn = torch.randn((T, H * P_), generator=g).to(dtype)
+    gated = ops.latent_gate(attn.cuda(), y_gpu, ncols - H, H, dv, P_)
+    assert rel_err(gated, K.latent_gate(attn, y_gpu.cpu(), ncols - H, H, dv, P_).double()) < tol
+    # one more token of each sequence: store, then attend over the cache
+    y1 = torch.randn((3, ncols), generator=g).to(dtype)
+    p1 = torch.tensor(lens, dtype=torch.int32)
+    s1 = torch.arange(3, dtype=torch.int32)
+    y1_gpu = y1.clone().cuda()
+    ops.latent_rope_store(y1_gpu, H, dn, dr, R, rot, cos_sin.cuda(), norm_w.cuda(), 1e-5, p1.cuda(), s1.cuda(),
+                          None, cache_gpu, table.cuda(), page, ring, False, ct_gpu)
+    K.latent_rope_store(y1, H, dn, dr, R, rot, cos_sin, norm_w, 1e-5, p1, s1, None, cache_ref, table, page, ring,
+                        False, ct_ref)
+    cache_gpu.copy_(cache_ref)
+    if transposed:
+        ct_gpu.copy_(ct_ref)
+    want = K.latent_attn_decode(y1_gpu.cpu(), w_uk, w_uv, ncols - H, cache_ref, table, page, ring, s1, p1 + 1, 0,
+                                H, dn, dr, R, dv, 0.2, window, 1).double()
+    for ct in ([None, ct_gpu] if transposed else [None]):
+        for nsplit in (1, 3, 7):
+            got = ops.latent_attn_decode(y1_gpu, w_uk.cuda(), w_uv.cuda(), ncols - H, cache_gpu, table.cuda(), page,
+                                         ring, s1.cuda(), (p1 + 1).cuda(), 0, H, dn, dr, R, dv, 0.2, window, nsplit, ct)
+            assert rel_err(got, want) < tol, (ct is not None, nsplit)
+
+
+
 @pytest.mark.parametrize("E", [96, 90, 2048])
 def test_norm_adds_a_pair_of_outputs(E):
     """x + (a + b) and the norm in one kernel, for all rows and for picked rows."""
