@@ -258,7 +258,7 @@ int illm_latent_absorb_q(const void* y, int dt, int ncols, const void* wuk, int 
 // One token per sequence over the latent cache: scores qa[b, h] . cache row, softmax over the
 // keys the token sees (all, or the last `window`), sums of latent rows.  Token b sees
 // seq_len[b] + len_more keys, itself included.  partial: float32 [B][H][nsplit][R + 4] = (sums,
-// max, weight, two unused) per range of keys.  R <= 512.
+// max, weight, two unused) per range of keys.  R <= 1024.
 int illm_latent_attn_decode(const float* qa, const void* cache, int dt, const int32_t* page_table,
                             int table_stride, int page_size, int ring, const int32_t* seq_slot,
                             const int32_t* seq_len, int len_more, float* partial, int nsplit, int B,

@@ -401,7 +401,8 @@ static int launch_latent_decode(int RC, dim3 grid, size_t smem, hipStream_t st, 
         case 1: GO(1);
         case 2: GO(2);
         case 4: GO(4);
-        default: GO(8);
+        case 8: GO(8);
+        default: GO(16);
     }
 #undef GO
 }
@@ -411,7 +412,7 @@ extern "C" int illm_latent_attn_decode(const float* qa, const void* cache, int d
                                        int ring, const int32_t* seq_slot, const int32_t* seq_len,
                                        int len_more, float* partial, int nsplit, int B, int H,
                                        int R, int dr, float scale, int window, void* stream) {
-    if (B < 0 || H <= 0 || R <= 0 || R > 512 || dr < 0 || nsplit < 1 || nsplit > 65535 ||
+    if (B < 0 || H <= 0 || R <= 0 || R > 1024 || dr < 0 || nsplit < 1 || nsplit > 65535 ||
         page_size <= 0 || page_size % 8 || table_stride <= 0 || !illm_dtype_ok(dt) || !partial)
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
@@ -420,7 +421,7 @@ extern "C" int illm_latent_attn_decode(const float* qa, const void* cache, int d
     const int groups = (H + HG - 1) / HG;
     if (groups > 65535) return ILLM_ERR_ARG;
     const int rc = (R + 63) / 64;
-    const int RC = rc <= 1 ? 1 : (rc <= 2 ? 2 : (rc <= 4 ? 4 : 8));
+    const int RC = rc <= 1 ? 1 : (rc <= 2 ? 2 : (rc <= 4 ? 4 : (rc <= 8 ? 8 : 16)));
     // row stride of a tile in LDS: lanes that read the same dim of different keys hit different banks
     int kstride;
     if (dt == ILLM_BF16) {
@@ -434,7 +435,7 @@ extern "C" int illm_latent_attn_decode(const float* qa, const void* cache, int d
     size_t smem = 0;
     for (; TK >= 8; TK >>= 1) {
         smem = (size_t)TK * 8 + (size_t)HG * D * 4 + (size_t)HG * TK * 4 + (size_t)TK * kstride * esz;
-        if (page_size % TK == 0 && smem <= 96 * 1024) break;
+        if (page_size % TK == 0 && smem <= 128 * 1024) break;
     }
     if (TK < 8) return ILLM_ERR_ARG;
     const dim3 grid(B, nsplit, groups);

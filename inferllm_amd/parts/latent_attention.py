@@ -45,8 +45,8 @@ class LatentAttention(Mixer):
         self.dn, self.dr, self.dv, self.R = int(head_dim), int(rot_dim), int(value_dim), int(rank)
         if min(self.E, self.H, self.dv, self.R) <= 0 or self.dn < 0 or self.dr < 0 or self.dn + self.dr <= 0:
             raise ValueError("latent attention: sizes must be positive")
-        if self.R > 512:
-            raise ValueError(f"latent attention: rank {self.R} is beyond the kernels' limit of 512")
+        if self.R > 1024:
+            raise ValueError(f"latent attention: rank {self.R} is beyond the kernels' limit of 1024")
         if max(self.dn + self.dr, self.dv) > 256:
             raise ValueError("latent attention: a head wider than 256 is beyond the attention kernels")
         self.scale, self.eps = float(softmax_scale), float(eps)
@@ -97,7 +97,7 @@ class LatentAttention(Mixer):
         self.w_up = _fuse([self.w_uk, self.w_uv])
         self.w_o = ops.decode_weight(self._take(tensors, "o").contiguous(), "plain", self.decode_copies)
         self.norm_w = self._take(tensors, "dkv_norm").contiguous()
-        self.transposed = (self.w_uk.dtype == torch.bfloat16 and self.R % 16 == 0
+        self.transposed = (self.w_uk.dtype == torch.bfloat16 and self.R % 16 == 0 and self.R <= 512
                            and (self.R + self.dr) % 8 == 0)
 
     def forward(self, h, ctx: StepContext, line, writes_cache, position):

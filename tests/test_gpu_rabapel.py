@@ -312,7 +312,7 @@ def test_architecture_is_chosen_by_config_and_refuses_what_it_lacks(tmp_path_fac
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,dn,dr,dv,R,rot,window", [(3, 16, 8, 24, 40, 8, 0), (16, 8, 16, 12, 64, 12, 70),
                                                      (5, 24, 32, 40, 48, 32, 33), (20, 16, 16, 16, 128, 16, 0),
-                                                     (1, 0, 8, 8, 16, 8, 65)])
+                                                     (1, 0, 8, 8, 16, 8, 65), (2, 8, 8, 8, 600, 8, 0)])
 def test_latent_kernels_alone(dtype, H, dn, dr, dv, R, rot, window):
     """Norm, rotation and store of the latent rows, the packed rows for prompts, the gate, and
     one token's attention over the paged latent cache (both kernels), against plain torch
