@@ -255,6 +255,16 @@ int illm_latent_gate(const void* attn, const void* y, int dt, int ncols, int gat
 int illm_latent_absorb_q(const void* y, int dt, int ncols, const void* wuk, int w_dt, void* qa,
                          int qa_dt, int B, int H, int dn, int dr, int R, void* stream);
 
+// Both in one launch, for rows that will walk the cache (single tokens): illm_latent_rope_store's
+// norm, rotation and store of the latent and the key part (no slot_len, no c_out / kr_out), and
+// illm_latent_absorb_q with the query's rot part rotated on its way (y keeps the unrotated query).
+int illm_latent_store_absorb(void* y, int dt, int ncols, int B, int H, int dn, int dr, int R, int rot,
+                             const float* cos_sin, int max_pos, const void* norm_w, int norm_dt,
+                             float eps, const int32_t* row_pos, const int32_t* row_slot, void* cache,
+                             const int32_t* page_table, int table_stride, int page_size, int ring,
+                             void* cache_t, const void* wuk, int w_dt, void* qa, int qa_dt,
+                             void* stream);
+
 // One token per sequence over the latent cache: scores qa[b, h] . cache row, softmax over the
 // keys the token sees (all, or the last `window`), sums of latent rows.  Token b sees
 // seq_len[b] + len_more keys, itself included.  partial: float32 [B][H][nsplit][R + 4] = (sums,

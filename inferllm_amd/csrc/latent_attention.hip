@@ -17,17 +17,16 @@
 // The latent is normed (float32 statistics), the shared key part and every head's rotated query
 // part are rotated in pairs (2i, 2i+1), i < rot/2, by the float32 table [max_pos][rot/2][2];
 // latent and key part go to the paged cache [page][row][R + dr] and to c_out / kr_out.
-__global__ void __launch_bounds__(256)
-latent_rope_store_kernel(void* __restrict__ y, int dt, int ncols, int H, int dn, int dr, int R,
-                         int rot, const float* __restrict__ cos_sin, int max_pos,
-                         const void* __restrict__ nw, int nw_dt, float eps,
-                         const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
-                         const int32_t* __restrict__ slot_len, void* __restrict__ cache,
-                         const int32_t* __restrict__ page_table, int table_stride, int page_size,
-                         int ring, void* __restrict__ c_out, void* __restrict__ kr_out,
-                         void* __restrict__ cache_t) {
+__device__ __forceinline__ void
+latent_store_row(const int t, void* __restrict__ y, int dt, int ncols, int H, int dn, int dr, int R,
+                 int rot, const float* __restrict__ cos_sin, int max_pos,
+                 const void* __restrict__ nw, int nw_dt, float eps,
+                 const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+                 const int32_t* __restrict__ slot_len, void* __restrict__ cache,
+                 const int32_t* __restrict__ page_table, int table_stride, int page_size,
+                 int ring, void* __restrict__ c_out, void* __restrict__ kr_out,
+                 void* __restrict__ cache_t, const bool rotate_q) {
     __shared__ float red[16];
-    const int t = blockIdx.x;
     int pos = row_pos[t];
     const size_t row = (size_t)t * ncols;
     const size_t down = row + (size_t)H * (dn + dr);
@@ -77,7 +76,7 @@ latent_rope_store_kernel(void* __restrict__ y, int dt, int ncols, int H, int dn,
         if (kr_out) st_f(kr_out, dt, (size_t)t * dr + e, v);
         if (store) st_f(cache, dt, dst + R + e, v);
     }
-    for (int u = threadIdx.x; u < H * half; u += blockDim.x) {
+    for (int u = threadIdx.x; rotate_q && u < H * half; u += blockDim.x) {
         const int h = u / half, i = u - h * half;
         const size_t base = row + (size_t)h * (dn + dr) + dn;
         const float c = cs[2 * i], s = cs[2 * i + 1];
@@ -85,6 +84,20 @@ latent_rope_store_kernel(void* __restrict__ y, int dt, int ncols, int H, int dn,
         st_f(y, dt, base + 2 * i, a * c - b * s);
         st_f(y, dt, base + 2 * i + 1, b * c + a * s);
     }
+}
+
+__global__ void __launch_bounds__(256)
+latent_rope_store_kernel(void* __restrict__ y, int dt, int ncols, int H, int dn, int dr, int R,
+                         int rot, const float* __restrict__ cos_sin, int max_pos,
+                         const void* __restrict__ nw, int nw_dt, float eps,
+                         const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+                         const int32_t* __restrict__ slot_len, void* __restrict__ cache,
+                         const int32_t* __restrict__ page_table, int table_stride, int page_size,
+                         int ring, void* __restrict__ c_out, void* __restrict__ kr_out,
+                         void* __restrict__ cache_t) {
+    latent_store_row(blockIdx.x, y, dt, ncols, H, dn, dr, R, rot, cos_sin, max_pos, nw, nw_dt, eps,
+                     row_pos, row_slot, slot_len, cache, page_table, table_stride, page_size, ring,
+                     c_out, kr_out, cache_t, true);
 }
 
 extern "C" int illm_latent_rope_store(void* y, int dt, int ncols, int T, int H, int dn, int dr,
@@ -170,15 +183,53 @@ extern "C" int illm_latent_gate(const void* attn, const void* y, int dt, int nco
 }
 
 // ---------------------------------------------------------------- queries against latent rows
+struct LatentStore {              // what the store of a row needs (see illm_latent_rope_store)
+    int rot, max_pos, nw_dt, table_stride, page_size, ring;
+    float eps;
+    const float* cos_sin;
+    const void* nw;
+    const int32_t* row_pos;
+    const int32_t* row_slot;
+    void* cache;
+    void* cache_t;
+    const int32_t* page_table;
+};
+
+// The rot part of a head's query in LDS (qs[dn ..]) rotated at the row's position.
+__device__ __forceinline__ void rotate_in_lds(float* qs, int dn, const LatentStore& st, int b) {
+    if (!st.cos_sin) return;
+    int pos = st.row_pos[b];
+    if (pos >= st.max_pos) pos = st.max_pos - 1;
+    const float* cs = st.cos_sin + (size_t)pos * st.rot;
+    for (int i = threadIdx.x; i < st.rot / 2; i += blockDim.x) {
+        const float c = cs[2 * i], s = cs[2 * i + 1];
+        const float a = qs[dn + 2 * i], v = qs[dn + 2 * i + 1];
+        qs[dn + 2 * i] = a * c - v * s;
+        qs[dn + 2 * i + 1] = v * c + a * s;
+    }
+    __syncthreads();
+}
+
 // qa[b, h] = [sum_d q[b, h, d] W_uk[h dn + d, :] (R) | q[b, h, dn:] (dr)], float32.  grid (B, H).
+// FUSED (grid (B, H + 1)): the query's rot part is rotated here, on its way (y keeps the
+// unrotated one), and block (b, H) norms, rotates and stores row b's latent and key part.
+template <bool FUSED>
 __global__ void __launch_bounds__(256)
-latent_absorb_q_kernel(const void* __restrict__ y, int dt, int ncols, const void* __restrict__ wuk,
-                       int w_dt, void* __restrict__ qa, int qa_dt, int H, int dn, int dr, int R) {
+latent_absorb_q_kernel(void* __restrict__ y, int dt, int ncols, const void* __restrict__ wuk,
+                       int w_dt, void* __restrict__ qa, int qa_dt, int H, int dn, int dr, int R,
+                       LatentStore st) {
     extern __shared__ float qs[];
     const int b = blockIdx.x, h = blockIdx.y;
+    if (FUSED && h == H) {
+        latent_store_row(b, y, dt, ncols, H, dn, dr, R, st.rot, st.cos_sin, st.max_pos, st.nw, st.nw_dt,
+                         st.eps, st.row_pos, st.row_slot, nullptr, st.cache, st.page_table,
+                         st.table_stride, st.page_size, st.ring, nullptr, nullptr, st.cache_t, false);
+        return;
+    }
     const size_t src = (size_t)b * ncols + (size_t)h * (dn + dr);
     for (int d = threadIdx.x; d < dn + dr; d += blockDim.x) qs[d] = ld_f(y, dt, src + d);
     __syncthreads();
+    if (FUSED) rotate_in_lds(qs, dn, st, b);
     const size_t dst = ((size_t)b * H + h) * (size_t)(R + dr);
     for (int r = threadIdx.x; r < R; r += blockDim.x) {
         float acc = 0.f;
@@ -192,17 +243,25 @@ latent_absorb_q_kernel(const void* __restrict__ y, int dt, int ncols, const void
 // The same for bfloat16 W_uk with R % 8 == 0 and R <= 512: a thread holds 8 neighbouring latent
 // dims (one 16-byte load a row of W_uk) and takes every (256 / (R / 8))-th plain dim; the groups'
 // sums are added through LDS in group order.
+template <bool FUSED>
 __global__ void __launch_bounds__(256)
-latent_absorb_q_bf16_kernel(const void* __restrict__ y, int dt, int ncols,
+latent_absorb_q_bf16_kernel(void* __restrict__ y, int dt, int ncols,
                             const bf16_t* __restrict__ wuk, void* __restrict__ qa, int qa_dt, int H,
-                            int dn, int dr, int R) {
+                            int dn, int dr, int R, LatentStore st) {
     extern __shared__ float sm[];
     float* qs = sm;                       // [dn + dr]
     float* part = sm + dn + dr;           // [groups][R]
     const int b = blockIdx.x, h = blockIdx.y;
+    if (FUSED && h == H) {
+        latent_store_row(b, y, dt, ncols, H, dn, dr, R, st.rot, st.cos_sin, st.max_pos, st.nw, st.nw_dt,
+                         st.eps, st.row_pos, st.row_slot, nullptr, st.cache, st.page_table,
+                         st.table_stride, st.page_size, st.ring, nullptr, nullptr, st.cache_t, false);
+        return;
+    }
     const size_t src = (size_t)b * ncols + (size_t)h * (dn + dr);
     for (int d = threadIdx.x; d < dn + dr; d += 256) qs[d] = ld_f(y, dt, src + d);
     __syncthreads();
+    if (FUSED) rotate_in_lds(qs, dn, st, b);
     const int per_row = R / 8, groups = 256 / per_row;
     const int c = threadIdx.x % per_row, g = threadIdx.x / per_row;
     float acc[8];
@@ -234,25 +293,58 @@ latent_absorb_q_bf16_kernel(const void* __restrict__ y, int dt, int ncols,
     for (int e = threadIdx.x; e < dr; e += 256) st_f(qa, qa_dt, dst + R + e, qs[dn + e]);
 }
 
-extern "C" int illm_latent_absorb_q(const void* y, int dt, int ncols, const void* wuk, int w_dt,
-                                    void* qa, int qa_dt, int B, int H, int dn, int dr, int R,
-                                    void* stream) {
-    if (B < 0 || H <= 0 || H > 65535 || dn < 0 || dr < 0 || R <= 0 || !illm_dtype_ok(dt) ||
-        !illm_dtype_ok(w_dt) || !illm_dtype_ok(qa_dt) || ncols < H * (dn + dr))
-        return ILLM_ERR_ARG;
-    if (B == 0) return ILLM_OK;
+template <bool FUSED>
+static int launch_absorb_q(void* y, int dt, int ncols, const void* wuk, int w_dt, void* qa, int qa_dt,
+                           int B, int H, int dn, int dr, int R, const LatentStore& st,
+                           hipStream_t stream) {
+    const dim3 grid(B, FUSED ? H + 1 : H);
     if (w_dt == ILLM_BF16 && R % 8 == 0 && R <= 512 && R >= 8) {
         const int groups = 256 / (R / 8);
         const size_t smem = ((size_t)(dn + dr) + (size_t)groups * R) * sizeof(float);
         if (smem <= 48 * 1024) {
-            hipLaunchKernelGGL(latent_absorb_q_bf16_kernel, dim3(B, H), dim3(256), smem,
-                               (hipStream_t)stream, y, dt, ncols, (const bf16_t*)wuk, qa, qa_dt, H, dn, dr, R);
+            hipLaunchKernelGGL(latent_absorb_q_bf16_kernel<FUSED>, grid, dim3(256), smem, stream, y, dt,
+                               ncols, (const bf16_t*)wuk, qa, qa_dt, H, dn, dr, R, st);
             return illm_launch_status();
         }
     }
-    hipLaunchKernelGGL(latent_absorb_q_kernel, dim3(B, H), dim3(256), (size_t)(dn + dr) * sizeof(float),
-                       (hipStream_t)stream, y, dt, ncols, wuk, w_dt, qa, qa_dt, H, dn, dr, R);
+    hipLaunchKernelGGL(latent_absorb_q_kernel<FUSED>, grid, dim3(256), (size_t)(dn + dr) * sizeof(float),
+                       stream, y, dt, ncols, wuk, w_dt, qa, qa_dt, H, dn, dr, R, st);
     return illm_launch_status();
+}
+
+extern "C" int illm_latent_absorb_q(const void* y, int dt, int ncols, const void* wuk, int w_dt,
+                                    void* qa, int qa_dt, int B, int H, int dn, int dr, int R,
+                                    void* stream) {
+    if (B < 0 || H <= 0 || H > 65534 || dn < 0 || dr < 0 || R <= 0 || !illm_dtype_ok(dt) ||
+        !illm_dtype_ok(w_dt) || !illm_dtype_ok(qa_dt) || ncols < H * (dn + dr))
+        return ILLM_ERR_ARG;
+    if (B == 0) return ILLM_OK;
+    LatentStore st = {};
+    return launch_absorb_q<false>((void*)y, dt, ncols, wuk, w_dt, qa, qa_dt, B, H, dn, dr, R, st,
+                                  (hipStream_t)stream);
+}
+
+extern "C" int illm_latent_store_absorb(void* y, int dt, int ncols, int B, int H, int dn, int dr,
+                                        int R, int rot, const float* cos_sin, int max_pos,
+                                        const void* norm_w, int norm_dt, float eps,
+                                        const int32_t* row_pos, const int32_t* row_slot, void* cache,
+                                        const int32_t* page_table, int table_stride, int page_size,
+                                        int ring, void* cache_t, const void* wuk, int w_dt, void* qa,
+                                        int qa_dt, void* stream) {
+    if (B < 0 || H <= 0 || H > 65534 || dn < 0 || dr < 0 || R <= 0 || !illm_dtype_ok(dt) ||
+        !illm_dtype_ok(w_dt) || !illm_dtype_ok(qa_dt) || !illm_dtype_ok(norm_dt) ||
+        ncols < H * (dn + dr) + R + dr || !row_pos)
+        return ILLM_ERR_ARG;
+    if (cos_sin && (rot <= 0 || rot > dr || (rot & 1) || max_pos <= 0)) return ILLM_ERR_ARG;
+    if (cache && (!page_table || !row_slot || page_size <= 0 || table_stride <= 0)) return ILLM_ERR_ARG;
+    if (B == 0) return ILLM_OK;
+    LatentStore st;
+    st.rot = rot; st.max_pos = max_pos; st.nw_dt = norm_dt; st.table_stride = table_stride;
+    st.page_size = page_size; st.ring = ring; st.eps = eps; st.cos_sin = cos_sin; st.nw = norm_w;
+    st.row_pos = row_pos; st.row_slot = row_slot; st.cache = cache; st.cache_t = cache_t;
+    st.page_table = page_table;
+    return launch_absorb_q<true>(y, dt, ncols, wuk, w_dt, qa, qa_dt, B, H, dn, dr, R, st,
+                                 (hipStream_t)stream);
 }
 
 // ---------------------------------------------------------------- one token over the latent cache

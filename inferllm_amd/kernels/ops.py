@@ -1130,29 +1130,72 @@ def latent_decode_mfma_fits(cache: torch.Tensor, cache_t: Optional[torch.Tensor]
             and (R + dr) % 8 == 0 and page_size % 32 == 0)
 
 
-def latent_attn_decode(y: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor, gate_off: int,
-                       cache: torch.Tensor, page_table: torch.Tensor, page_size: int, ring: int,
-                       seq_slot: torch.Tensor, seq_len: torch.Tensor, len_more: int, H: int, dn: int,
-                       dr: int, R: int, dv: int, scale: float, window: int, nsplit: int,
-                       cache_t: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """One token per sequence over the latent cache, never building a head's keys or values:
-    queries are taken through W_uk first, the weighted sums of latent rows through W_uv after,
-    then the head's output gate.  y [B, ...] = [q (rotated) | down | gate]; token b sees
-    seq_len[b] + len_more keys of the sequence in seq_slot[b], itself included; returns [B, H dv]."""
-    _gpu(y, w_uk, w_uv, cache, page_table, seq_slot, seq_len)
+def latent_absorb_q(y: torch.Tensor, w_uk: torch.Tensor, H: int, dn: int, dr: int, R: int,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """qa [B, H, R + dr] = [W_uk,h^T q_h | q_h's rot part] of the (already rotated) queries in y:
+    what a head's query looks like against latent rows.  float32 sums; bfloat16 for the
+    matrix-core kernel, of whose product it is an operand."""
+    _gpu(y, w_uk)
     B = y.shape[0]
-    _i32(page_table); _i32(seq_slot, B); _i32(seq_len, B)
-    _need(w_uk.shape == (H * dn, R) and w_uv.shape == (H * dv, R), "latent_attn_decode: W_uk / W_uv")
-    _need(cache.dim() == 3 and cache.shape[1:] == (page_size, R + dr) and cache.dtype == y.dtype,
-          "latent_attn_decode: cache shape or dtype")
-    # the matrix-core kernel takes the queries in bfloat16 (they are an operand of its product)
-    qa = torch.empty((B, H, R + dr), dtype=torch.bfloat16 if cache_t is not None else torch.float32,
-                     device=y.device)
+    _need(w_uk.shape == (H * dn, R), "latent_absorb_q: W_uk [H dn, R]")
+    qa = torch.empty((B, H, R + dr), dtype=out_dtype, device=y.device)
     _check(_lib().illm_latent_absorb_q(_p(y), _code(y), y.shape[1], _p(w_uk), _code(w_uk), _p(qa),
                                        _code(qa), B, H, dn, dr, R, _stream()), "latent_absorb_q")
+    return qa
+
+
+def latent_store_absorb(y: torch.Tensor, H: int, dn: int, dr: int, R: int, rot: int,
+                        cos_sin: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
+                        row_pos: torch.Tensor, row_slot: torch.Tensor, cache: torch.Tensor,
+                        page_table: torch.Tensor, page_size: int, ring: int, w_uk: torch.Tensor,
+                        out_dtype: torch.dtype, cache_t: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`latent_rope_store` (without the rows' copies) and `latent_absorb_q` in one launch, for rows
+    that will walk the cache: the latent and key part of every row are normed, rotated and stored,
+    and qa is made from the queries with their rot part rotated on the way (y keeps them unrotated)."""
+    _gpu(y, cos_sin, norm_w, row_pos, row_slot, cache, page_table, w_uk, cache_t)
+    B, ncols = y.shape
+    _i32(row_pos, B); _i32(row_slot, B); _i32(page_table)
+    _need(ncols >= H * (dn + dr) + R + dr and norm_w.shape == (R,) and w_uk.shape == (H * dn, R),
+          "latent_store_absorb: shapes")
+    max_pos = 0
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.shape[1] * 2 == rot
+              and cos_sin.shape[2] == 2 and rot <= dr,
+              "latent_store_absorb: angle table must be float32 [max_pos, rot/2, 2], rot <= dr")
+        max_pos = cos_sin.shape[0]
+    _need(cache.dtype == y.dtype and cache.dim() == 3 and cache.shape[1:] == (page_size, R + dr)
+          and page_table.dim() == 2, "latent_store_absorb: cache shape or dtype")
+    _need(cache_t is None or (cache_t.dtype == y.dtype and cache_t.shape == (cache.shape[0], R, page_size, 1)),
+          "latent_store_absorb: the transposed copy must be [pages, R, page_size, 1]")
+    qa = torch.empty((B, H, R + dr), dtype=out_dtype, device=y.device)
+    _check(_lib().illm_latent_store_absorb(
+        _p(y), _code(y), ncols, B, H, dn, dr, R, rot, _p(cos_sin), max_pos, _p(norm_w), _code(norm_w),
+        ctypes.c_float(eps), _p(row_pos), _p(row_slot), _p(cache), _p(page_table), page_table.shape[1],
+        page_size, ring, _p(cache_t), _p(w_uk), _code(w_uk), _p(qa), _code(qa), _stream()),
+        "latent_store_absorb")
+    return qa
+
+
+def latent_attn_decode(qa: torch.Tensor, y: torch.Tensor, w_uv: torch.Tensor, gate_off: int,
+                       cache: torch.Tensor, page_table: torch.Tensor, page_size: int, ring: int,
+                       seq_slot: torch.Tensor, seq_len: torch.Tensor, len_more: int, H: int, dr: int,
+                       R: int, dv: int, scale: float, window: int, nsplit: int,
+                       cache_t: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per sequence over the latent cache, never building a head's keys or values: the
+    queries qa [B, H, R + dr] have been taken through W_uk (`latent_absorb_q`), the weighted sums of
+    latent rows go through W_uv after, then the head's output gate (y[:, gate_off + h]).  Token b
+    sees seq_len[b] + len_more keys of the sequence in seq_slot[b], itself included.  With the
+    transposed copy `cache_t` (and qa in bfloat16) both products run on the matrix cores.
+    Returns [B, H dv]."""
+    _gpu(qa, y, w_uv, cache, page_table, seq_slot, seq_len, cache_t)
+    B = y.shape[0]
+    _i32(page_table); _i32(seq_slot, B); _i32(seq_len, B)
+    _need(w_uv.shape == (H * dv, R) and qa.shape == (B, H, R + dr), "latent_attn_decode: W_uv or qa")
+    _need(cache.dim() == 3 and cache.shape[1:] == (page_size, R + dr) and cache.dtype == y.dtype,
+          "latent_attn_decode: cache shape or dtype")
     partial = torch.empty((B, H, nsplit, R + 4), dtype=torch.float32, device=y.device)
     if cache_t is not None:
-        _need(latent_decode_mfma_fits(cache, cache_t, R, dr, page_size) and
+        _need(latent_decode_mfma_fits(cache, cache_t, R, dr, page_size) and qa.dtype == torch.bfloat16 and
               cache_t.shape == (cache.shape[0], R, page_size, 1) and cache_t.is_contiguous(),
               "latent_attn_decode: the transposed copy is not taken")
         _check(_lib().illm_latent_attn_decode_mfma(
@@ -1160,8 +1203,9 @@ def latent_attn_decode(y: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor, 
             _p(seq_slot), _p(seq_len), len_more, _p(partial), nsplit, B, H, R, dr,
             ctypes.c_float(scale), window, _stream()), f"latent_attn_decode_mfma (latent {R}+{dr})")
     else:
+        _need(qa.dtype == torch.float32, "latent_attn_decode: float32 queries")
         _check(_lib().illm_latent_attn_decode(
-        _p(qa), _p(cache), _code(cache), _p(page_table), page_table.shape[1], page_size, ring,
+            _p(qa), _p(cache), _code(cache), _p(page_table), page_table.shape[1], page_size, ring,
             _p(seq_slot), _p(seq_len), len_more, _p(partial), nsplit, B, H, R, dr, ctypes.c_float(scale),
             window, _stream()), f"latent_attn_decode (latent {R}+{dr})")
     out = torch.empty((B, H * dv), dtype=y.dtype, device=y.device)

@@ -113,12 +113,11 @@ class LatentAttention(Mixer):
         if not self.gated:
             y = torch.cat([y, y.new_full((y.shape[0], H), 30.0)], dim=1)       # sigmoid(30) = 1
         whole = ctx.prefill and not ctx.continues
-        c, kr = ops.latent_rope_store(
-            y, H, dn, dr, R, rot, table, self.norm_w, self.eps, ctx.row_pos, ctx.row_slot,
-            ctx.cache.slot_len if ctx.prefill else None, cache if writes_cache else None,
-            group.table, group.page_size, group.ring, want_rows=whole,
-            cache_t=cache_t if writes_cache else None)
         if whole:
+            c, kr = ops.latent_rope_store(
+                y, H, dn, dr, R, rot, table, self.norm_w, self.eps, ctx.row_pos, ctx.row_slot,
+                ctx.cache.slot_len, cache if writes_cache else None, group.table, group.page_size,
+                group.ring, want_rows=True, cache_t=cache_t if writes_cache else None)
             if writes_cache:
                 ctx.exchange[("latent_rows", line)] = (c, kr)
             else:
@@ -129,6 +128,18 @@ class LatentAttention(Mixer):
                                  self.scale, window)
             o = ops.latent_gate(a, y, self.gate_off, H, dv, P)
         else:
+            # rows that walk the cache: the store of the row and the queries against latent rows
+            # in one launch (a run that only reads the line rotates its queries and stores nothing)
+            qa_dtype = torch.bfloat16 if cache_t is not None else torch.float32
+            if writes_cache:
+                qa = ops.latent_store_absorb(y, H, dn, dr, R, rot, table, self.norm_w, self.eps,
+                                             ctx.row_pos, ctx.row_slot, cache, group.table,
+                                             group.page_size, group.ring, self.w_uk, qa_dtype, cache_t)
+            else:
+                ops.latent_rope_store(y, H, dn, dr, R, rot, table, self.norm_w, self.eps, ctx.row_pos,
+                                      ctx.row_slot, None, None, group.table, group.page_size,
+                                      group.ring, want_rows=False)
+                qa = ops.latent_absorb_q(y, self.w_uk, H, dn, dr, R, qa_dtype)
             longest = min(ctx.max_len, window) if window else ctx.max_len
             nsplit = ops.latent_decode_splits(y.shape[0], H, longest, mfma=cache_t is not None)
             if ctx.prefill:
@@ -136,7 +147,7 @@ class LatentAttention(Mixer):
                 slots, lens, more = ctx.row_slot, ctx.row_pos, 1
             else:
                 slots, lens, more = ctx.seq_slot, ctx.seq_len, 0
-            o = ops.latent_attn_decode(y, self.w_uk, self.w_uv, self.gate_off, cache, group.table,
-                                       group.page_size, group.ring, slots, lens, more, H, dn, dr,
-                                       R, dv, self.scale, window, nsplit, cache_t)
+            o = ops.latent_attn_decode(qa, y, self.w_uv, self.gate_off, cache, group.table,
+                                       group.page_size, group.ring, slots, lens, more, H, dr, R, dv,
+                                       self.scale, window, nsplit, cache_t)
         return ops.linear(o, self.w_o)

@@ -320,20 +320,39 @@ def latent_decode_mfma_fits(cache, cache_t, R, dr, page_size):
     return False
 
 
-def latent_attn_decode(y, w_uk, w_uv, gate_off, cache, page_table, page_size, ring, seq_slot, seq_len,
-                       len_more, H, dn, dr, R, dv, scale, window, nsplit, cache_t=None):
+def latent_absorb_q(y, w_uk, H, dn, dr, R, out_dtype):
+    B = y.shape[0]
+    q = y[:, :H * (dn + dr)].to(F64).reshape(B, H, dn + dr)
+    wk = w_uk.to(F64).reshape(H, dn, R)
+    return torch.cat([torch.einsum("bhd,hdr->bhr", q[:, :, :dn], wk), q[:, :, dn:]], dim=-1).to(out_dtype)
+
+
+def latent_store_absorb(y, H, dn, dr, R, rot, cos_sin, norm_w, eps, row_pos, row_slot, cache, page_table,
+                        page_size, ring, w_uk, out_dtype, cache_t=None):
+    rotated = y.clone()                                # y itself keeps the unrotated queries
+    latent_rope_store(rotated, H, dn, dr, R, rot, cos_sin, norm_w, eps, row_pos, row_slot, None, cache,
+                      page_table, page_size, ring, False, cache_t)
+    if y.dtype != torch.float32:
+        # the rotated part is not rounded on its way: take it from the unrounded rotation
+        wide = y.to(F64)
+        latent_rope_store(wide, H, dn, dr, R, rot, cos_sin, norm_w, eps, row_pos, row_slot, None, None,
+                          page_table, page_size, ring, False)
+        rotated = wide
+    return latent_absorb_q(rotated, w_uk, H, dn, dr, R, out_dtype)
+
+
+def latent_attn_decode(qa, y, w_uv, gate_off, cache, page_table, page_size, ring, seq_slot, seq_len,
+                       len_more, H, dr, R, dv, scale, window, nsplit, cache_t=None):
     B = y.shape[0]
     out = torch.zeros((B, H * dv), dtype=y.dtype)
-    wk, wv = w_uk.to(F64).reshape(H, dn, R), w_uv.to(F64).reshape(H, dv, R)
+    wv = w_uv.to(F64).reshape(H, dv, R)
     for b in range(B):
         slot, L = int(seq_slot[b]), int(seq_len[b]) + len_more
         lo = max(0, L - window) if window and window > 0 else 0
         rows = torch.stack([cache[cache_offsets(page_table, slot, p, page_size, ring)] for p in range(lo, L)]).to(F64)
-        q = y[b, :H * (dn + dr)].to(F64).reshape(H, dn + dr)
         gate = torch.sigmoid(y[b, gate_off:gate_off + H].to(F64))
         for h in range(H):
-            qa = torch.cat([q[h, :dn] @ wk[h], q[h, dn:]])
-            p = torch.softmax((rows @ qa) * scale, dim=0)
+            p = torch.softmax((rows @ qa[b, h].to(F64)) * scale, dim=0)
             out[b, h * dv:(h + 1) * dv] = ((wv[h] @ (p @ rows[:, :R])) * gate[h]).to(y.dtype)
     return out
 
@@ -383,6 +402,7 @@ def patch(monkeypatch):
                  "linear_add_fits",
                  "attn_prefill", "attn_prefill_paged", "decode_splits", "attn_decode", "argmax", "sample",
                  "sum_rows", "relu_squared", "latent_rope_store", "latent_pack", "latent_gate",
-                 "latent_decode_splits", "latent_decode_mfma_fits", "latent_attn_decode",
+                 "latent_decode_splits", "latent_decode_mfma_fits", "latent_attn_decode", "latent_absorb_q",
+                 "latent_store_absorb",
                  "few_outputs_f32", "moe_route", "moe_experts", "moe_combine"):
         monkeypatch.setattr(ops, name, globals()[name])

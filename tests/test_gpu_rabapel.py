@@ -358,26 +358,32 @@ def test_latent_kernels_alone(dtype, H, dn, dr, dv, R, rot, window):
     attn = torch.randn((T, H * P_), generator=g).to(dtype)
     gated = ops.latent_gate(attn.cuda(), y_gpu, ncols - H, H, dv, P_)
     assert rel_err(gated, K.latent_gate(attn, y_gpu.cpu(), ncols - H, H, dv, P_).double()) < tol
-    # one more token of each sequence: store, then attend over the cache
+    # one more token of each sequence: store and queries in one launch, then the walk over the cache
     y1 = torch.randn((3, ncols), generator=g).to(dtype)
     p1 = torch.tensor(lens, dtype=torch.int32)
     s1 = torch.arange(3, dtype=torch.int32)
     y1_gpu = y1.clone().cuda()
-    ops.latent_rope_store(y1_gpu, H, dn, dr, R, rot, cos_sin.cuda(), norm_w.cuda(), 1e-5, p1.cuda(), s1.cuda(),
-                          None, cache_gpu, table.cuda(), page, ring, False, ct_gpu)
-    K.latent_rope_store(y1, H, dn, dr, R, rot, cos_sin, norm_w, 1e-5, p1, s1, None, cache_ref, table, page, ring,
-                        False, ct_ref)
-    cache_gpu.copy_(cache_ref)
-    if transposed:
-        ct_gpu.copy_(ct_ref)
-    want = K.latent_attn_decode(y1_gpu.cpu(), w_uk, w_uv, ncols - H, cache_ref, table, page, ring, s1, p1 + 1, 0,
-                                H, dn, dr, R, dv, 0.2, window, 1).double()
-    for ct in ([None, ct_gpu] if transposed else [None]):
+    for qa_dtype in ([torch.float32, torch.bfloat16] if transposed else [torch.float32]):
+        ct = ct_gpu if qa_dtype == torch.bfloat16 else None
+        qa_g = ops.latent_store_absorb(y1_gpu, H, dn, dr, R, rot, cos_sin.cuda(), norm_w.cuda(), 1e-5, p1.cuda(),
+                                       s1.cuda(), cache_gpu, table.cuda(), page, ring, w_uk.cuda(), qa_dtype, ct_gpu)
+        qa_r = K.latent_store_absorb(y1, H, dn, dr, R, rot, cos_sin, norm_w, 1e-5, p1, s1, cache_ref, table, page,
+                                     ring, w_uk, qa_dtype, ct_ref)
+        assert torch.equal(y1_gpu.cpu(), y1)                      # the rows keep their unrotated queries
+        assert rel_err(qa_g, qa_r.double()) < (tol if qa_dtype == torch.float32 else 2e-2)
+        assert float((cache_gpu.double().cpu() - cache_ref.double()).abs().max()) <= tol * max(1.0, float(cache_ref.double().abs().max()))
+        cache_gpu.copy_(cache_ref)
+        if transposed:
+            ct_gpu.copy_(ct_ref)
+        want = K.latent_attn_decode(qa_g.cpu(), y1, w_uv, ncols - H, cache_ref, table, page, ring, s1, p1 + 1, 0,
+                                    H, dr, R, dv, 0.2, window, 1).double()
         for nsplit in (1, 3, 7):
-            got = ops.latent_attn_decode(y1_gpu, w_uk.cuda(), w_uv.cuda(), ncols - H, cache_gpu, table.cuda(), page,
-                                         ring, s1.cuda(), (p1 + 1).cuda(), 0, H, dn, dr, R, dv, 0.2, window, nsplit, ct)
-            assert rel_err(got, want) < tol, (ct is not None, nsplit)
-
+            got = ops.latent_attn_decode(qa_g, y1_gpu, w_uv.cuda(), ncols - H, cache_gpu, table.cuda(), page, ring,
+                                         s1.cuda(), (p1 + 1).cuda(), 0, H, dr, R, dv, 0.2, window, nsplit, ct)
+            assert rel_err(got, want) < tol, (qa_dtype, nsplit)
+    # the queries' product alone (rows whose queries are rotated already)
+    qa2 = ops.latent_absorb_q(y_gpu[:5].contiguous(), w_uk.cuda(), H, dn, dr, R, torch.float32)
+    assert rel_err(qa2, K.latent_absorb_q(y_gpu[:5].cpu(), w_uk, H, dn, dr, R, torch.float32).double()) < tol
 
 
 @pytest.mark.parametrize("E", [96, 90, 2048])
