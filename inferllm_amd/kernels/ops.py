@@ -1250,10 +1250,63 @@ MOE_MFMA_FROM = 0        # (token, choice) pairs an expert on average from which
                          # K took 253 + 166 us for 64 tokens, bound by its sums across lanes)
 
 
-def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+def _moe_tiling(dtype: torch.dtype, E: int, F: int, NP: int, n_exp: int):
+    """(on the matrix cores?, rows a tile, upper bound of tiles) for NP (token, choice) pairs."""
+    # many pairs an expert (prompts): tiles of up to 64 rows; few (single tokens): tiles of 16 rows
+    # on the matrix cores, or of 8 rows with a wave a column (float32, odd sizes)
+    per_expert = NP / max(1, n_exp)
+    mfma = dtype == torch.bfloat16 and E % 32 == 0 and F % 32 == 0 and per_expert >= MOE_MFMA_FROM
+    rows = (64 if per_expert >= 48 else 32 if per_expert >= 24 else 16) if mfma else _lib().illm_moe_tile_rows()
+    return mfma, rows, max(1, min(NP, NP // rows + n_exp))
+
+
+def _moe_group(idx: torch.Tensor, n_exp: int, dtype: torch.dtype, E: int, F: int):
+    NP = idx.numel()
+    mfma, rows, max_tiles = _moe_tiling(dtype, E, F, NP, n_exp)
+    order = torch.empty((NP,), dtype=torch.int32, device=idx.device)
+    tiles = torch.empty((3 * max_tiles + 1,), dtype=torch.int32, device=idx.device)
+    _check(_lib().illm_moe_group(_p(idx), NP, n_exp, _p(order), _p(tiles), max_tiles, rows,
+                                 _stream()), "moe_group")
+    return order, tiles, max_tiles, rows, mfma
+
+
+def moe_plan(h: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int,
+             w_gate_up: Optional[torch.Tensor]):
+    """A routed layer's plan for the rows h: (idx, weight, grouped).  idx, weight [T, top] as
+    `moe_route` gives them for the router's float32 outputs h . w_router^T; grouped: the pairs
+    grouped by expert for `moe_experts` (None without stacked experts).  Few tokens: one launch
+    for all three steps, with the same results."""
+    _gpu(h, w_router, correction)
+    T, E = h.shape
+    NE = w_router.shape[0]
+    n_exp = w_gate_up.shape[0] if w_gate_up is not None else 0
+    small = _lib().illm_moe_plan_small_tokens()
+    if 0 < T <= small and (T * NE + T * top) * 4 <= 40 * 1024 and n_exp > 0:
+        _need(w_router.dtype == torch.float32 and w_router.shape[1] == E, "moe_plan: float32 router [outputs, E]")
+        _need(correction is None or correction.shape == (NE,), "moe_plan: correction [outputs]")
+        F = w_gate_up.shape[1] // 2
+        NP = T * top
+        mfma, rows, max_tiles = _moe_tiling(h.dtype, E, F, NP, n_exp)
+        idx = torch.empty((T, top), dtype=torch.int32, device=h.device)
+        wt = torch.empty((T, top), dtype=torch.float32, device=h.device)
+        order = torch.empty((NP,), dtype=torch.int32, device=h.device)
+        tiles = torch.empty((3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
+        _check(_lib().illm_moe_plan_small(
+            _p(h), _code(h), _p(w_router), _p(correction),
+            _code(correction) if correction is not None else 0, T, NE, E, top, n_exp, _p(idx), _p(wt),
+            _p(order), _p(tiles), max_tiles, rows, _stream()), "moe_plan_small")
+        return idx, wt, (order, tiles, max_tiles, rows, mfma)
+    idx, wt = moe_route(few_outputs_f32(h, w_router), correction, top)
+    grouped = _moe_group(idx, n_exp, h.dtype, E, w_gate_up.shape[1] // 2) if n_exp else None
+    return idx, wt, grouped
+
+
+def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
+                grouped=None) -> torch.Tensor:
     """Y [T * top, E]: for every (token, choice) pair whose choice is one of the stacked experts
     (w_gate_up [experts, 2 F, E] = [gate | up], w_down [experts, E, F]) the expert's
-    down(silu(gate h) * (up h)); rows of other pairs are not written."""
+    down(silu(gate h) * (up h)); rows of other pairs are not written.  `grouped`: the pairs by
+    expert as `moe_plan` left them (else they are grouped here)."""
     _gpu(h, idx, w_gate_up, w_down)
     _i32(idx)
     T, E = h.shape
@@ -1264,16 +1317,7 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gate_up: torch.Tensor, w_d
           "moe_experts: shapes or dtypes")
     NP = T * top
     F = F2 // 2
-    # many pairs an expert (prompts): tiles of up to 64 rows on the matrix cores; few (single
-    # tokens): tiles of 8 rows, a wave a column, which reads an expert's matrices once
-    per_expert = NP / max(1, n_exp)
-    mfma = h.dtype == torch.bfloat16 and E % 32 == 0 and F % 32 == 0 and per_expert >= MOE_MFMA_FROM
-    rows = (64 if per_expert >= 48 else 32 if per_expert >= 24 else 16) if mfma else _lib().illm_moe_tile_rows()
-    max_tiles = max(1, min(NP, NP // rows + n_exp))
-    order = torch.empty((NP,), dtype=torch.int32, device=h.device)
-    tiles = torch.empty((3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
-    _check(_lib().illm_moe_group(_p(idx), NP, n_exp, _p(order), _p(tiles), max_tiles, rows,
-                                 _stream()), "moe_group")
+    order, tiles, max_tiles, rows, mfma = grouped if grouped is not None else _moe_group(idx, n_exp, h.dtype, E, F)
     act = torch.empty((NP, F), dtype=h.dtype, device=h.device)
     y = torch.empty((NP, E), dtype=h.dtype, device=h.device)
     if mfma:

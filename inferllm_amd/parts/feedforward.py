@@ -172,9 +172,8 @@ class RoutedExperts(FeedForward):
                 self.w_sg = take("shared.sg").reshape(-1).contiguous()
 
     def forward(self, h, ctx: StepContext):
-        z = ops.few_outputs_f32(h, self.w_router)
-        idx, weight = ops.moe_route(z, self.correction, self.top)
-        y = ops.moe_experts(h, idx, self.w_gate_up, self.w_down) if self.n_real else None
+        idx, weight, grouped = ops.moe_plan(h, self.w_router, self.correction, self.top, self.w_gate_up)
+        y = ops.moe_experts(h, idx, self.w_gate_up, self.w_down, grouped) if self.n_real else None
         shared = None
         if self.Fs:
             shared = ops.linear(ops.gate_up_silu(h, self.w_shared_gate_up), self.w_shared_down)

@@ -369,7 +369,12 @@ def moe_route(z, correction, top):
     return idx.to(torch.int32), torch.gather(s, 1, idx).to(torch.float32)
 
 
-def moe_experts(h, idx, w_gate_up, w_down):
+def moe_plan(h, w_router, correction, top, w_gate_up):
+    idx, wt = moe_route(few_outputs_f32(h, w_router), correction, top)
+    return idx, wt, None
+
+
+def moe_experts(h, idx, w_gate_up, w_down, grouped=None):
     T, top = idx.shape
     F = w_gate_up.shape[1] // 2
     y = torch.zeros((T * top, h.shape[1]), dtype=h.dtype)
@@ -404,5 +409,5 @@ def patch(monkeypatch):
                  "sum_rows", "relu_squared", "latent_rope_store", "latent_pack", "latent_gate",
                  "latent_decode_splits", "latent_decode_mfma_fits", "latent_attn_decode", "latent_absorb_q",
                  "latent_store_absorb",
-                 "few_outputs_f32", "moe_route", "moe_experts", "moe_combine"):
+                 "few_outputs_f32", "moe_route", "moe_plan", "moe_experts", "moe_combine"):
         monkeypatch.setattr(ops, name, globals()[name])

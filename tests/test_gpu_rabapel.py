@@ -420,6 +420,34 @@ def test_router_kernel(n_out, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T", [1, 3, 8, 9, 40])
+def test_router_product_choice_and_grouping_in_one_launch_or_three(dtype, T):
+    """Few tokens take one launch for the router's product, the choice and the grouping: the same
+    choices and weights as the three kernels give (the same bits), and every pair in its expert's group."""
+    from inferllm_amd.kernels import ops
+    g = torch.Generator().manual_seed(T)
+    E, NE, n_real, top, F = 96, 11, 8, 3, 32
+    h = torch.randn((T, E), generator=g).to(dtype).cuda()
+    w = torch.randn((NE, E), generator=g).cuda()
+    corr = (torch.randn((NE,), generator=g) * 0.05).to(dtype).cuda()
+    wgu = torch.zeros((n_real, 2 * F, E), dtype=dtype).cuda()
+    idx, wt, (order, tiles, max_tiles, rows, _) = ops.moe_plan(h, w, corr, top, wgu)
+    idx3, wt3 = ops.moe_route(ops.few_outputs_f32(h, w), corr, top)
+    assert torch.equal(idx, idx3) and torch.equal(wt, wt3)
+    want = torch.topk(torch.softmax(h.double().cpu() @ w.double().cpu().T, -1) + corr.double().cpu(), top).indices
+    assert torch.equal(idx.cpu().long(), want)
+    n_tiles = int(tiles[3 * max_tiles])
+    seen = []
+    for i in range(n_tiles):
+        e, first, n = (int(v) for v in tiles[3 * i:3 * i + 3])
+        assert 0 < n <= rows
+        pairs = order[first:first + n].cpu().tolist()
+        assert all(int(idx.view(-1)[p]) == e for p in pairs)
+        seen += pairs
+    assert sorted(seen) == [p for p in range(T * top) if int(idx.view(-1)[p]) < n_real]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("E,F,n_real,n_id,top,T", [(64, 40, 5, 2, 3, 37), (90, 30, 2, 0, 1, 9),
                                                    (128, 96, 12, 4, 2, 300), (96, 64, 6, 1, 2, 3),
                                                    (160, 32, 4, 0, 3, 40), (256, 128, 3, 1, 2, 700),
