@@ -307,13 +307,6 @@ int illm_moe_tile_rows(void);
 int illm_moe_group(const int32_t* idx, int NP, int NEr, int32_t* order, int32_t* tiles,
                    int max_tiles, int tile_rows, void* stream);
 
-// illm_few_outputs_f32, illm_moe_route and illm_moe_group in one launch for up to
-// illm_moe_plan_small_tokens() tokens (x [T, K], w [NE, K] float32): the same results.
-int illm_moe_plan_small_tokens(void);
-int illm_moe_plan_small(const void* x, int x_dt, const float* w, const void* corr, int corr_dt, int T,
-                        int NE, int K, int top, int NEr, int32_t* idx, float* wt, int32_t* order,
-                        int32_t* tiles, int max_tiles, int tile_rows, void* stream);
-
 // Y[p] = X[p / x_div] . W[e_p]^T for every grouped pair p (W [experts][N][K]); gated: W
 // [experts][2 N][K] = [gate | up] rows and Y[p] = silu(X Wg^T) * (X Wu^T).  Y [NP, N] of dt.
 int illm_moe_rows(const void* X, int x_div, const void* W, int dt, int gated, const int32_t* order,

@@ -223,64 +223,6 @@ moe_group_kernel(const int32_t* __restrict__ idx, int NP, int NEr, int32_t* __re
     moe_group_pairs(idx, NP, NEr, order, tiles, max_tiles, tile_rows);
 }
 
-// Router product, choice and grouping of up to MOE_PLAN_TOKENS tokens in one block of 16 waves
-// (single tokens: three launches less a routed layer).  The sums run as in few_outputs_f32 (lanes
-// over K, four neighbouring k a lane where K % 4 == 0), so a token's outputs are the same bits
-// either way.
-#define MOE_PLAN_TOKENS 8
-__global__ void __launch_bounds__(1024)
-moe_plan_small_kernel(const void* __restrict__ x, int x_dt, const float* __restrict__ w,
-                      const void* __restrict__ corr, int corr_dt, int T, int NE, int K, int top,
-                      int NEr, int32_t* __restrict__ idx, float* __restrict__ wt,
-                      int32_t* __restrict__ order, int32_t* __restrict__ tiles, int max_tiles,
-                      int tile_rows) {
-    extern __shared__ float zs[];                      // [T][NE] logits, then [T * top] choices
-    int32_t* idx_s = (int32_t*)(zs + (size_t)T * NE);
-    const int wv = wave_index(), lane = threadIdx.x & 63;
-    for (int p = wv; p < T * NE; p += 16) {
-        const int t = p / NE, e = p - t * NE;
-        const float* wr = w + (size_t)e * K;
-        float acc = 0.f;
-        if (K % 4 == 0) {
-#pragma unroll 2
-            for (int k = lane * 4; k < K; k += 256) {
-                const float4 a = *(const float4*)(wr + k);
-                const float4 b = ld4_f32(x, x_dt, (size_t)t * K + k);
-                acc += b.x * a.x; acc += b.y * a.y; acc += b.z * a.z; acc += b.w * a.w;
-            }
-        } else {
-#pragma unroll 4
-            for (int k = lane; k < K; k += 64) acc += ld_f(x, x_dt, (size_t)t * K + k) * wr[k];
-        }
-        acc = wave_sum(acc);
-        if (lane == 0) zs[p] = acc;
-    }
-    __syncthreads();
-    if (wv < T)
-        moe_route_row(zs + (size_t)wv * NE, corr, corr_dt, NE, top, idx + (size_t)wv * top,
-                      wt + (size_t)wv * top, idx_s + wv * top);
-    __syncthreads();
-    moe_group_pairs(idx_s, T * top, NEr, order, tiles, max_tiles, tile_rows);
-}
-
-extern "C" int illm_moe_plan_small_tokens(void) { return MOE_PLAN_TOKENS; }
-
-extern "C" int illm_moe_plan_small(const void* x, int x_dt, const float* w, const void* corr,
-                                   int corr_dt, int T, int NE, int K, int top, int NEr,
-                                   int32_t* idx, float* wt, int32_t* order, int32_t* tiles,
-                                   int max_tiles, int tile_rows, void* stream) {
-    if (T <= 0 || T > MOE_PLAN_TOKENS || NE <= 0 || NE > 64 * MOE_EPL || top <= 0 || top > NE ||
-        K <= 0 || NEr < 0 || NEr > MOE_MAX_EXPERTS || max_tiles < 0 || tile_rows <= 0 ||
-        !illm_dtype_ok(x_dt) || (corr && !illm_dtype_ok(corr_dt)))
-        return ILLM_ERR_ARG;
-    const size_t smem = ((size_t)T * NE + (size_t)T * top) * 4;
-    if (smem > 40 * 1024) return ILLM_ERR_ARG;
-    hipLaunchKernelGGL(moe_plan_small_kernel, dim3(1), dim3(1024), smem, (hipStream_t)stream, x, x_dt,
-                       w, corr, corr_dt, T, NE, K, top, NEr, idx, wt, order, tiles, max_tiles,
-                       tile_rows);
-    return illm_launch_status();
-}
-
 extern "C" int illm_moe_tile_rows(void) { return MOE_TILE; }
 
 extern "C" int illm_moe_group(const int32_t* idx, int NP, int NEr, int32_t* order, int32_t* tiles,

@@ -1274,28 +1274,9 @@ def moe_plan(h: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch
              w_gate_up: Optional[torch.Tensor]):
     """A routed layer's plan for the rows h: (idx, weight, grouped).  idx, weight [T, top] as
     `moe_route` gives them for the router's float32 outputs h . w_router^T; grouped: the pairs
-    grouped by expert for `moe_experts` (None without stacked experts).  Few tokens: one launch
-    for all three steps, with the same results."""
-    _gpu(h, w_router, correction)
-    T, E = h.shape
-    NE = w_router.shape[0]
+    grouped by expert for `moe_experts` (None without stacked experts)."""
+    E = h.shape[1]
     n_exp = w_gate_up.shape[0] if w_gate_up is not None else 0
-    small = _lib().illm_moe_plan_small_tokens()
-    if 0 < T <= small and (T * NE + T * top) * 4 <= 40 * 1024 and n_exp > 0:
-        _need(w_router.dtype == torch.float32 and w_router.shape[1] == E, "moe_plan: float32 router [outputs, E]")
-        _need(correction is None or correction.shape == (NE,), "moe_plan: correction [outputs]")
-        F = w_gate_up.shape[1] // 2
-        NP = T * top
-        mfma, rows, max_tiles = _moe_tiling(h.dtype, E, F, NP, n_exp)
-        idx = torch.empty((T, top), dtype=torch.int32, device=h.device)
-        wt = torch.empty((T, top), dtype=torch.float32, device=h.device)
-        order = torch.empty((NP,), dtype=torch.int32, device=h.device)
-        tiles = torch.empty((3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
-        _check(_lib().illm_moe_plan_small(
-            _p(h), _code(h), _p(w_router), _p(correction),
-            _code(correction) if correction is not None else 0, T, NE, E, top, n_exp, _p(idx), _p(wt),
-            _p(order), _p(tiles), max_tiles, rows, _stream()), "moe_plan_small")
-        return idx, wt, (order, tiles, max_tiles, rows, mfma)
     idx, wt = moe_route(few_outputs_f32(h, w_router), correction, top)
     grouped = _moe_group(idx, n_exp, h.dtype, E, w_gate_up.shape[1] // 2) if n_exp else None
     return idx, wt, grouped

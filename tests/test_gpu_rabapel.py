@@ -421,9 +421,9 @@ def test_router_kernel(n_out, top):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T", [1, 3, 8, 9, 40])
-def test_router_product_choice_and_grouping_in_one_launch_or_three(dtype, T):
-    """Few tokens take one launch for the router's product, the choice and the grouping: the same
-    choices and weights as the three kernels give (the same bits), and every pair in its expert's group."""
+def test_router_product_choice_and_grouping(dtype, T):
+    """A routed layer's plan: the choices and weights of the router's float32 product, and every
+    (token, choice) pair in its expert's group, in tiles of no more rows than said."""
     from inferllm_amd.kernels import ops
     g = torch.Generator().manual_seed(T)
     E, NE, n_real, top, F = 96, 11, 8, 3, 32
