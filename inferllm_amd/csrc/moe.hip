@@ -659,7 +659,7 @@ extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int g
 }
 
 // ---------------------------------------------------------------- weighted sum
-// grid (tokens, chunks of 1024 columns): out[t] = sum_k wt[t, k] * (idx[t, k] < NEr ? Y[t top + k] : h[t])
+// grid (tokens, chunks of 256 columns): out[t] = sum_k wt[t, k] * (idx[t, k] < NEr ? Y[t top + k] : h[t])
 //                                         (+ sigmoid(h[t] . sg) * shared[t]), float32.
 #define MOE_COMBINE_TOP 16                          // choices held in registers (more: read again)
 __global__ void __launch_bounds__(256)
@@ -686,8 +686,8 @@ moe_combine_kernel(const void* __restrict__ h, int dt, const int32_t* __restrict
             gate = 1.0f / (1.0f + expf(-d));
         }
     }
-    const int i_end = min(E, (int)(blockIdx.y + 1) * 1024);
-    for (int i = blockIdx.y * 1024 + threadIdx.x; i < i_end; i += 256) {
+    const int i_end = min(E, (int)(blockIdx.y + 1) * 256);
+    for (int i = blockIdx.y * 256 + threadIdx.x; i < i_end; i += 256) {
         const float hv = ld_f(h, dt, t * E + i);
         float acc = 0.f;
         if (top <= MOE_COMBINE_TOP) {
@@ -713,10 +713,10 @@ extern "C" int illm_moe_combine(const void* h, int dt, const int32_t* idx, const
                                 const void* Y, const void* shared, const void* sg, int sg_dt,
                                 float* out, int T, int E, int top, int NEr, void* stream) {
     if (T < 0 || E <= 0 || top <= 0 || !illm_dtype_ok(dt) || (sg && !illm_dtype_ok(sg_dt)) ||
-        (E + 1023) / 1024 > 65535)
+        (E + 255) / 256 > 65535)
         return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(T, (E + 1023) / 1024), dim3(256), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(T, (E + 255) / 256), dim3(256), 0, (hipStream_t)stream,
                        h, dt, idx, wt, Y, shared, sg, sg_dt, out, E, top, NEr);
     return illm_launch_status();
 }
