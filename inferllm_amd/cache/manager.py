@@ -81,9 +81,11 @@ class KVSpec:
 
 @dataclass(frozen=True)
 class StateSpec:
-    """Fixed-size state per sequence for one cache line: shape and dtype."""
+    """Fixed-size state per sequence for one cache line: shape and dtype (None: the engine's).
+    A mixer that keeps several such tensors names them: a dict name -> StateSpec in place of one
+    StateSpec, read back as a dict of tensors."""
     shape: Tuple[int, ...]
-    dtype: torch.dtype = torch.float32
+    dtype: Optional[torch.dtype] = torch.float32
 
 
 class KVGroup:
@@ -227,8 +229,11 @@ class CacheManager:
         # most tokens a sequence may bring to a step that reads the cache (None: any number)
         self.step_limit: Optional[int] = min(limits) if limits else None
         self._group_of: Dict[int, KVGroup] = {l: g for g in self.groups for l in g.lines}
-        self.states: Dict[int, torch.Tensor] = {
-            line: torch.zeros((max_slots + 1,) + tuple(s.shape), dtype=s.dtype, device=device)
+        def state(s: StateSpec) -> torch.Tensor:
+            return torch.zeros((max_slots + 1,) + tuple(s.shape), dtype=s.dtype or dtype, device=device)
+        # line -> tensor [slot, *shape], or name -> tensor for a mixer that keeps several
+        self.states: Dict[int, object] = {
+            line: ({name: state(one) for name, one in s.items()} if isinstance(s, dict) else state(s))
             for line, s in state_lines.items()}
         self.len_host = torch.zeros(max_slots + 1, dtype=torch.int32)
         self._len = self.len_host.numpy()       # the same memory; element access costs far less
@@ -241,9 +246,15 @@ class CacheManager:
         slot = self.slots.alloc()
         self._len[slot] = 0
         self._len_dirty = True
-        for t in self.states.values():
+        for t in self._state_tensors():
             t[slot].zero_()
         return slot
+
+    def _state_tensors(self) -> List[torch.Tensor]:
+        out: List[torch.Tensor] = []
+        for t in self.states.values():
+            out.extend(t.values() if isinstance(t, dict) else [t])
+        return out
 
     def free_slot(self, slot: int) -> None:
         self.slots.free(slot)           # raises if not held
@@ -344,7 +355,9 @@ class CacheManager:
         i = g.line_index(line)
         return {name: t[i] for name, t in g.tensors.items()}, g
 
-    def state_line(self, line: int) -> Optional[torch.Tensor]:
+    def state_line(self, line: int):
+        """The state of a cache line: a tensor [slot, *shape], a dict of such tensors by name if
+        its mixer keeps several, or None."""
         return self.states.get(line)
 
     def tokens_held(self) -> int:

@@ -28,14 +28,19 @@ class PartSpec:
 
 @dataclass
 class LayerSpec:
-    """A block: its arrangement ("pre_norm", "parallel") and the parts it is made of.  An
-    arrangement with one norm (both parts read its rows) has no `feed_forward_norm`."""
+    """A block: its arrangement ("pre_norm", "parallel", "hyper_connections") and the parts it
+    is made of.  An arrangement with one norm (both parts read its rows) has no
+    `feed_forward_norm`.  An arrangement with constants or tensors of its own (the weights with
+    which several residual streams are mixed) takes them as `block_params` and `block_tensors`
+    (own parameter name -> checkpoint tensor name)."""
     block: str
     mixer: PartSpec
     feed_forward: PartSpec
     mixer_norm: PartSpec
     feed_forward_norm: Optional[PartSpec] = None
     position: Optional[PartSpec] = None
+    block_params: Dict[str, Any] = field(default_factory=dict)
+    block_tensors: Dict[str, str] = field(default_factory=dict)
 
 
 @dataclass

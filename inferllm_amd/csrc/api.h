@@ -22,6 +22,9 @@ int illm_embed_scaled(const int32_t* tokens, const void* table, int table_dt, fl
 // out[i] = float32(a[i]) + float32(b[i]): the two outputs of a block whose parts read the same rows.
 int illm_sum_rows(const void* a, int a_dt, const void* b, int b_dt, float* out, size_t n,
                   void* stream);
+// out[i] = sa float32(a[i]) + sb float32(b[i]).
+int illm_sum_rows_scaled(const void* a, int a_dt, float sa, const void* b, int b_dt, float sb,
+                         float* out, size_t n, void* stream);
 
 // out[i] = max(x[i], 0)^2.
 int illm_relu_squared(const void* x, void* out, int dt, size_t n, void* stream);
@@ -296,8 +299,9 @@ int illm_few_outputs_f32(const void* x, int x_dt, const float* w, float* z, int 
 
 // idx, wt [T, top]: the `top` outputs of z [T, NE] (float32) with the largest softmax(z) + corr
 // (corr may be null), in falling order, and their softmax values.  NE <= 512.
+// score_kind 0: softmax over all outputs; 1: every output's sigmoid.
 int illm_moe_route(const float* z, const void* corr, int corr_dt, int T, int NE, int top,
-                   int32_t* idx, float* wt, void* stream);
+                   int32_t* idx, float* wt, int score_kind, void* stream);
 
 // order [NP]: the pairs whose choice is below NEr, grouped by choice; tiles [3 max_tiles + 1]:
 // (expert, first place in order, rows <= tile_rows) per tile and, last, their number.
@@ -309,19 +313,69 @@ int illm_moe_group(const int32_t* idx, int NP, int NEr, int32_t* order, int32_t*
 
 // Y[p] = X[p / x_div] . W[e_p]^T for every grouped pair p (W [experts][N][K]); gated: W
 // [experts][2 N][K] = [gate | up] rows and Y[p] = silu(X Wg^T) * (X Wu^T).  Y [NP, N] of dt.
+// act_kind (gated only) 0: silu(g) * u; 1: with g = min(g, limit), u = clamp(u, -limit, limit):
+// g * sigmoid(1.702 g) * (u + 1).  row_w (may be null; gated only): a weight per pair that
+// multiplies the pair's X row (applied to the two products, which is the same).
 int illm_moe_rows(const void* X, int x_div, const void* W, int dt, int gated, const int32_t* order,
-                  const int32_t* tiles, int max_tiles, void* Y, int N, int K, void* stream);
+                  const int32_t* tiles, int max_tiles, void* Y, int N, int K, int act_kind,
+                  float limit, const float* row_w, void* stream);
 
 // The same for bfloat16 with K % 32 == 0 and tiles of up to 16, 32 or 64 rows, on the matrix cores.
 int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int gated, int tile_rows,
                        const int32_t* order, const int32_t* tiles, int max_tiles, void* Y, int N,
-                       int K, void* stream);
+                       int K, int act_kind, float limit, const float* row_w, void* stream);
 
 // out[t] = sum_k wt[t, k] * (idx[t, k] < NEr ? Y[t top + k] : h[t]) (+ g * shared[t], with
-// g = sigmoid(h[t] . sg), or 1 if sg is null; shared may be null), float32 [T, E].
+// g = sigmoid(h[t] . sg), or 1 if sg is null; shared may be null), float32 [T, E].  wt null: every
+// weight 1.
 int illm_moe_combine(const void* h, int dt, const int32_t* idx, const float* wt, const void* Y,
                      const void* shared, const void* sg, int sg_dt, float* out, int T, int E, int top,
                      int NEr, void* stream);
+
+// ---- several residual streams (streams.hip)
+// x float32 [T, S, E].  If y1: x_t <- sum_s mix[s, t] x_s + outw[t] (ya y1 (+ yb y2)) for every
+// stream t (written back unless row_idx); then u = sum_s read[s] x_s (read null: weights 1) and
+// h[r] = u / sqrt(mean(u^2) + eps) * w for every row (or those row_idx names).  S <= 8.
+int illm_stream_mix_norm(float* x, int S, const void* y1, int y1_dt, float ya, const void* y2,
+                         int y2_dt, float yb, const float* mix, const float* outw,
+                         const float* read, const void* w, int w_dt, void* h, int h_dt,
+                         const int32_t* row_idx, int rows, int E, float eps, void* stream);
+// out[t, s, :] = table[tokens[t], :] * scale for every stream s < S.
+int illm_embed_streams(const int32_t* tokens, const void* table, int table_dt, float* out, int T,
+                       int E, int V, int S, float scale, void* stream);
+
+// ---- the gated delta rule (delta_rule.hip)
+int illm_delta_prepare(const void* P, int p_dt, int p_stride, int b_off, const void* A, int a_dt,
+                       int a_stride, int a_off, const float* conv_w, int taps, const void* tail,
+                       int tail_dt, const int32_t* row_slot, const float* a_log,
+                       const float* dt_bias, float* qn, float* kn, float* vv, float* beta,
+                       float* dec, int T, int G, int H, int dk, int dv, int DW, void* stream);
+int illm_delta_conv_tail(const void* P, int p_dt, int p_stride, void* tail, int tail_dt,
+                         const int32_t* cu, const int32_t* seq_slot, int n_seqs, int C, int taps,
+                         void* stream);
+int illm_delta_scan(const float* qn, const float* kn, const float* vv, const float* beta,
+                    const float* dec, int DW, float* state, const int32_t* cu,
+                    const int32_t* seq_slot, float* o, int n_seqs, int G, int H, int dk, int dv,
+                    void* stream);
+int illm_delta_finish(const float* o, const void* w, int w_dt, const void* Z, int z_dt, int z_stride,
+                      int z_off, int gate_kind, void* out, int out_dt, int T, int H, int dv,
+                      float eps, void* stream);
+
+// ---- attention with a soft cap on the scores and value heads of their own width (attention_capped.hip)
+int illm_kv_store2(const void* rows, int dt, int row_len, int k_off, int v_off,
+                   const int32_t* row_pos, const int32_t* row_slot, void* kcache, void* vcache,
+                   const int32_t* page_table, int table_stride, int page_size, int ring, int T,
+                   int nkv, int dk, int dv, void* stream);
+int illm_attn_cap_rows(const void* q, int q_stride, void* out, int dt, const int32_t* cu,
+                       const int32_t* seq_slot, const int32_t* seq_start, const void* kcache,
+                       const void* vcache, const int32_t* page_table, int table_stride,
+                       int page_size, int ring, int n_seqs, int max_rows, int nh, int nkv, int dk,
+                       int dv, float scale, float cap, int window, void* stream);
+int illm_attn_cap_decode(const void* q, int q_stride, void* out, int dt, const void* kcache,
+                         const void* vcache, const int32_t* page_table, int table_stride,
+                         int page_size, int ring, const int32_t* seq_slot, const int32_t* seq_len,
+                         float* partial, int nsplit, int B, int nh, int nkv, int dk, int dv,
+                         float scale, float cap, int window, void* stream);
 
 #ifdef __cplusplus
 }

@@ -53,6 +53,22 @@ extern "C" int illm_sum_rows(const void* a, int a_dt, const void* b, int b_dt, f
     return illm_launch_status();
 }
 
+__global__ void sum_rows_scaled_kernel(const void* __restrict__ a, int a_dt, float sa,
+                                       const void* __restrict__ b, int b_dt, float sb,
+                                       float* __restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = sa * ld_f(a, a_dt, i) + sb * ld_f(b, b_dt, i);
+}
+
+extern "C" int illm_sum_rows_scaled(const void* a, int a_dt, float sa, const void* b, int b_dt,
+                                    float sb, float* out, size_t n, void* stream) {
+    if (!illm_dtype_ok(a_dt) || !illm_dtype_ok(b_dt)) return ILLM_ERR_ARG;
+    if (n == 0) return ILLM_OK;
+    hipLaunchKernelGGL(sum_rows_scaled_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, a, a_dt, sa, b, b_dt, sb, out, n);
+    return illm_launch_status();
+}
+
 __global__ void relu_squared_kernel(const void* __restrict__ x, void* __restrict__ out, int dt,
                                     size_t n) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

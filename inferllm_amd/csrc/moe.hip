@@ -101,12 +101,27 @@ extern "C" int illm_few_outputs_f32(const void* x, int x_dt, const float* w, flo
     return illm_launch_status();
 }
 
-// One wave per token: s = softmax(z) over all NE outputs (float32), choice score = s + correction,
+// Scores of a router's outputs: their softmax, or every output's sigmoid.
+#define MOE_SCORE_SOFTMAX 0
+#define MOE_SCORE_SIGMOID 1
+// What an expert does with its gate and up products: silu(gate) * up, or with both clamped
+// (gate from above, up on both sides, at `limit`) gate * sigmoid(1.702 gate) * (up + 1).
+#define MOE_ACT_SILU 0
+#define MOE_ACT_CLAMPED 1
+__device__ __forceinline__ float moe_act(float gate, float up, int act_kind, float limit) {
+    if (act_kind == MOE_ACT_SILU) return (gate / (1.0f + expf(-gate))) * up;
+    gate = fminf(gate, limit);
+    up = fminf(fmaxf(up, -limit), limit);
+    return (gate / (1.0f + expf(-1.702f * gate))) * (up + 1.0f);
+}
+
+// One wave per token: s = the scores of all NE outputs (float32), choice score = s + correction,
 // the `top` largest choice scores (lowest index on ties) in falling order; weights are s.
 #define MOE_EPL 8                                   // outputs a lane holds: up to 512 experts
 __device__ __forceinline__ void
 moe_route_row(const float* zr, const void* __restrict__ corr, int corr_dt, int NE, int top,
-              int32_t* __restrict__ idx_row, float* __restrict__ wt_row, int32_t* idx_copy) {
+              int32_t* __restrict__ idx_row, float* __restrict__ wt_row, int32_t* idx_copy,
+              int score_kind) {
     const int lane = threadIdx.x & 63;
     float s[MOE_EPL], c[MOE_EPL];
     float mx = -INFINITY;
@@ -127,7 +142,8 @@ moe_route_row(const float* zr, const void* __restrict__ corr, int corr_dt, int N
 #pragma unroll
     for (int i = 0; i < MOE_EPL; ++i) {
         const int e = lane + 64 * i;
-        s[i] = s[i] / sum;
+        // softmax over all outputs, or every output's own sigmoid
+        s[i] = score_kind == MOE_SCORE_SIGMOID ? (e < NE ? 1.0f / (1.0f + expf(-zr[e])) : 0.f) : s[i] / sum;
         c[i] = e < NE ? s[i] + (corr ? ld_f(corr, corr_dt, e) : 0.f) : -INFINITY;
     }
     for (int k = 0; k < top; ++k) {
@@ -158,18 +174,18 @@ moe_route_row(const float* zr, const void* __restrict__ corr, int corr_dt, int N
 
 __global__ void __launch_bounds__(64)
 moe_route_kernel(const float* __restrict__ z, const void* __restrict__ corr, int corr_dt, int NE,
-                 int top, int32_t* __restrict__ idx, float* __restrict__ wt) {
+                 int top, int32_t* __restrict__ idx, float* __restrict__ wt, int score_kind) {
     const size_t t = blockIdx.x;
-    moe_route_row(z + t * NE, corr, corr_dt, NE, top, idx + t * top, wt + t * top, nullptr);
+    moe_route_row(z + t * NE, corr, corr_dt, NE, top, idx + t * top, wt + t * top, nullptr, score_kind);
 }
 
 extern "C" int illm_moe_route(const float* z, const void* corr, int corr_dt, int T, int NE, int top,
-                              int32_t* idx, float* wt, void* stream) {
-    if (T < 0 || NE <= 0 || NE > 64 * MOE_EPL || top <= 0 || top > NE || (corr && !illm_dtype_ok(corr_dt)))
+                              int32_t* idx, float* wt, int score_kind, void* stream) {
+    if ((score_kind != MOE_SCORE_SOFTMAX && score_kind != MOE_SCORE_SIGMOID) || T < 0 || NE <= 0 || NE > 64 * MOE_EPL || top <= 0 || top > NE || (corr && !illm_dtype_ok(corr_dt)))
         return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
     hipLaunchKernelGGL(moe_route_kernel, dim3(T), dim3(64), 0, (hipStream_t)stream, z, corr, corr_dt,
-                       NE, top, idx, wt);
+                       NE, top, idx, wt, score_kind);
     return illm_launch_status();
 }
 
@@ -262,7 +278,8 @@ template <int DT, int V, bool GATED>
 __global__ void __launch_bounds__(256)
 moe_rows_kernel(const void* __restrict__ X, int x_div, const void* __restrict__ W,
                 const int32_t* __restrict__ order, const int32_t* __restrict__ tiles, int max_tiles,
-                void* __restrict__ Y, int N, int K, int cols_per_block) {
+                void* __restrict__ Y, int N, int K, int cols_per_block, int act_kind, float limit,
+                const float* __restrict__ row_w) {
     const int tile = blockIdx.x;
     if (tile >= tiles[3 * (size_t)max_tiles]) return;
     const int e = tiles[3 * (size_t)tile], first = tiles[3 * (size_t)tile + 1];
@@ -316,8 +333,9 @@ moe_rows_kernel(const void* __restrict__ X, int x_div, const void* __restrict__ 
                         // the products take the activations' type before the activation, as a
                         // product of its own would leave them
                         float gate = v, upv = lane ? g[1][r] : g[0][r];
+                        if (row_w) { gate *= row_w[pair[r]]; upv *= row_w[pair[r]]; }   // W (w x) = w (W x)
                         if (DT == ILLM_BF16) { gate = bf16_to_f32(f32_to_bf16(gate)); upv = bf16_to_f32(f32_to_bf16(upv)); }
-                        v = (gate / (1.0f + expf(-gate))) * upv;
+                        v = moe_act(gate, upv, act_kind, limit);
                     }
                     if (DT == ILLM_BF16) ((bf16_t*)Y)[(size_t)pair[r] * N + col + lane] = f32_to_bf16(v);
                     else ((float*)Y)[(size_t)pair[r] * N + col + lane] = v;
@@ -329,8 +347,9 @@ moe_rows_kernel(const void* __restrict__ X, int x_div, const void* __restrict__ 
 
 extern "C" int illm_moe_rows(const void* X, int x_div, const void* W, int dt, int gated,
                              const int32_t* order, const int32_t* tiles, int max_tiles, void* Y,
-                             int N, int K, void* stream) {
-    if (x_div <= 0 || N <= 0 || K <= 0 || max_tiles < 0 || max_tiles > 2147483647 / 3 ||
+                             int N, int K, int act_kind, float limit, const float* row_w,
+                             void* stream) {
+    if ((act_kind != MOE_ACT_SILU && act_kind != MOE_ACT_CLAMPED) || x_div <= 0 || N <= 0 || K <= 0 || max_tiles < 0 || max_tiles > 2147483647 / 3 ||
         !illm_dtype_ok(dt))
         return ILLM_ERR_ARG;
     if (max_tiles == 0) return ILLM_OK;
@@ -340,7 +359,7 @@ extern "C" int illm_moe_rows(const void* X, int x_div, const void* W, int dt, in
     hipStream_t st = (hipStream_t)stream;
 #define GO(DT_, V_, G_)                                                                          \
     hipLaunchKernelGGL((moe_rows_kernel<DT_, V_, G_>), grid, dim3(256), 0, st, X, x_div, W, order, \
-                       tiles, max_tiles, Y, N, K, cols)
+                       tiles, max_tiles, Y, N, K, cols, act_kind, limit, row_w)
     if (dt == ILLM_BF16) {
         if (K % 8 == 0) { if (gated) GO(ILLM_BF16, 8, true); else GO(ILLM_BF16, 8, false); }
         else { if (gated) GO(ILLM_BF16, 1, true); else GO(ILLM_BF16, 1, false); }
@@ -366,7 +385,8 @@ template <int MT, int NT, bool GATED, bool AHEAD, int KU>
 __global__ void __launch_bounds__(256)
 moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __restrict__ W,
                      const int32_t* __restrict__ order, const int32_t* __restrict__ tiles,
-                     int max_tiles, bf16_t* __restrict__ Y, int N, int K) {
+                     int max_tiles, bf16_t* __restrict__ Y, int N, int K, int act_kind, float limit,
+                     const float* __restrict__ row_w) {
     const int tile = blockIdx.x;
     if (tile >= tiles[3 * (size_t)max_tiles]) return;
     const int e = tiles[3 * (size_t)tile], first = tiles[3 * (size_t)tile + 1];
@@ -487,9 +507,10 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __re
                 if (col >= N) continue;
                 float v = a[nt][mt][i];
                 if (GATED) {
-                    const float gate = bf16_to_f32(f32_to_bf16(a[nt][mt][i]));
-                    const float upv = bf16_to_f32(f32_to_bf16(g[nt][mt][i]));
-                    v = (gate / (1.0f + expf(-gate))) * upv;
+                    const float rw = row_w ? row_w[pair[mt]] : 1.0f;          // W (w x) = w (W x)
+                    const float gate = bf16_to_f32(f32_to_bf16(a[nt][mt][i] * rw));
+                    const float upv = bf16_to_f32(f32_to_bf16(g[nt][mt][i] * rw));
+                    v = moe_act(gate, upv, act_kind, limit);
                 }
                 Y[(size_t)pair[mt] * N + col] = f32_to_bf16(v);
             }
@@ -505,7 +526,8 @@ template <int NT, bool GATED>
 __global__ void __launch_bounds__(256)
 moe_rows_mfma_lds_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* __restrict__ W,
                          const int32_t* __restrict__ order, const int32_t* __restrict__ tiles,
-                         int max_tiles, bf16_t* __restrict__ Y, int N, int K) {
+                         int max_tiles, bf16_t* __restrict__ Y, int N, int K, int act_kind,
+                         float limit, const float* __restrict__ row_w) {
     constexpr int MT = 4;
     __shared__ uint4 xs[2][64 * 8];
     const int tile = blockIdx.x;
@@ -605,9 +627,10 @@ moe_rows_mfma_lds_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* 
                 if (col >= N) continue;
                 float v = a[nt][mt][i];
                 if (GATED) {
-                    const float gate = bf16_to_f32(f32_to_bf16(a[nt][mt][i]));
-                    const float upv = bf16_to_f32(f32_to_bf16(g[nt][mt][i]));
-                    v = (gate / (1.0f + expf(-gate))) * upv;
+                    const float rw = row_w ? row_w[pair[mt]] : 1.0f;          // W (w x) = w (W x)
+                    const float gate = bf16_to_f32(f32_to_bf16(a[nt][mt][i] * rw));
+                    const float upv = bf16_to_f32(f32_to_bf16(g[nt][mt][i] * rw));
+                    v = moe_act(gate, upv, act_kind, limit);
                 }
                 Y[(size_t)pair[mt] * N + col] = f32_to_bf16(v);
             }
@@ -616,8 +639,9 @@ moe_rows_mfma_lds_kernel(const bf16_t* __restrict__ X, int x_div, const bf16_t* 
 
 extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int gated, int tile_rows,
                                   const int32_t* order, const int32_t* tiles, int max_tiles,
-                                  void* Y, int N, int K, void* stream) {
-    if (x_div <= 0 || N <= 0 || K <= 0 || K % 32 || max_tiles < 0 || max_tiles > 2147483647 / 3 ||
+                                  void* Y, int N, int K, int act_kind, float limit,
+                                  const float* row_w, void* stream) {
+    if ((act_kind != MOE_ACT_SILU && act_kind != MOE_ACT_CLAMPED) || x_div <= 0 || N <= 0 || K <= 0 || K % 32 || max_tiles < 0 || max_tiles > 2147483647 / 3 ||
         (tile_rows != 16 && tile_rows != 32 && tile_rows != 64))
         return ILLM_ERR_ARG;
     if (max_tiles == 0) return ILLM_OK;
@@ -628,10 +652,10 @@ extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int g
         if (grid.y > 65535) return ILLM_ERR_ARG;
         if (gated)
             hipLaunchKernelGGL((moe_rows_mfma_lds_kernel<2, true>), grid, dim3(256), 0, st, (const bf16_t*)X,
-                               x_div, (const bf16_t*)W, order, tiles, max_tiles, (bf16_t*)Y, N, K);
+                               x_div, (const bf16_t*)W, order, tiles, max_tiles, (bf16_t*)Y, N, K, act_kind, limit, row_w);
         else
             hipLaunchKernelGGL((moe_rows_mfma_lds_kernel<4, false>), grid, dim3(256), 0, st, (const bf16_t*)X,
-                               x_div, (const bf16_t*)W, order, tiles, max_tiles, (bf16_t*)Y, N, K);
+                               x_div, (const bf16_t*)W, order, tiles, max_tiles, (bf16_t*)Y, N, K, act_kind, limit, row_w);
         return illm_launch_status();
     }
 #define GO(MT_, NT_, G_, KU_)                                                                      \
@@ -640,7 +664,7 @@ extern "C" int illm_moe_rows_mfma(const void* X, int x_div, const void* W, int g
         if (grid.y > 65535) return ILLM_ERR_ARG;                                                   \
         hipLaunchKernelGGL((moe_rows_mfma_kernel<MT_, NT_, G_, (MT_ * NT_ <= 16), KU_>), grid, dim3(256), 0, st, \
                            (const bf16_t*)X, x_div, (const bf16_t*)W, order, tiles, max_tiles,     \
-                           (bf16_t*)Y, N, K);                                                      \
+                           (bf16_t*)Y, N, K, act_kind, limit, row_w);                              \
     } while (0)
     if (tile_rows == 16 && (long)max_tiles * ((N + 255) / 256) < 512) {
         // few tiles (single tokens): 16 columns a wave, so that more waves share the reading
@@ -674,7 +698,7 @@ moe_combine_kernel(const void* __restrict__ h, int dt, const int32_t* __restrict
 #pragma unroll
     for (int k = 0; k < MOE_COMBINE_TOP; ++k) {
         ce[k] = k < top ? idx[t * top + k] : 0;
-        cw[k] = k < top ? wt[t * top + k] : 0.f;
+        cw[k] = k < top ? (wt ? wt[t * top + k] : 1.f) : 0.f;
     }
     float gate = 0.f;
     if (shared) {
@@ -701,7 +725,7 @@ moe_combine_kernel(const void* __restrict__ h, int dt, const int32_t* __restrict
         } else {
             for (int k = 0; k < top; ++k) {
                 const int e = idx[t * top + k];
-                acc += wt[t * top + k] * (e < NEr ? ld_f(Y, dt, (t * top + k) * E + i) : hv);
+                acc += (wt ? wt[t * top + k] : 1.f) * (e < NEr ? ld_f(Y, dt, (t * top + k) * E + i) : hv);
             }
         }
         if (shared) acc += gate * ld_f(shared, dt, t * E + i);

@@ -19,7 +19,7 @@ from ..cache.slots import CacheError, CacheFull
 from ..config.registry import config_from_dict, load_config
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
-from ..weights.loader import load_named_tensors
+from ..weights.loader import load_named_tensors, stored_shapes
 from ..weights.random_init import random_tensors
 from .generate import GenerationLoop, GenerationStats
 from .model import DecoderModel
@@ -131,6 +131,10 @@ class Engine:
         then run on the float32 multiply-add kernel, at twice the memory and a fraction of the
         speed (a warning says so)."""
         config = load_config(model_dir)
+        if hasattr(config, "with_tensor_shapes"):
+            # a design may leave sizes to its tensors' shapes (a low rank, say): the configuration
+            # takes them from the folder before anything is built
+            config = config.with_tensor_shapes(stored_shapes(model_dir))
         model = DecoderModel(config.to_spec())
         dt = parse_dtype(dtype)
         tensors = load_named_tensors(model_dir, model.wants(), dt, device,

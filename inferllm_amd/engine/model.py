@@ -39,7 +39,9 @@ class DecoderModel:
                 mixer_norm=build_part("norm", ls.mixer_norm),
                 feed_forward_norm=(build_part("norm", ls.feed_forward_norm)
                                    if ls.feed_forward_norm is not None else None),
-                position=position))
+                position=position,
+                **({"tensors": ls.block_tensors, **ls.block_params}
+                   if ls.block_tensors or ls.block_params else {})))
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
         self.schedule = list(spec.schedule)

@@ -96,12 +96,18 @@ def _check(rc: int, what: str) -> None:
 
 
 # ------------------------------------------------------------------ rows
-def embed(tokens: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
-    """float32 [T, E] rows of `table` [V, E] at int32 `tokens` [T], times `scale`."""
+def embed(tokens: torch.Tensor, table: torch.Tensor, scale: float = 1.0, copies: int = 0) -> torch.Tensor:
+    """float32 [T, E] rows of `table` [V, E] at int32 `tokens` [T], times `scale`; with `copies`
+    > 0, [T, copies, E]: the row once for every residual stream."""
     _gpu(tokens, table)
     _i32(tokens)
     _need(table.dim() == 2 and tokens.dim() == 1, "embed: tokens [T], table [V, E]")
     T, (V, E) = tokens.numel(), table.shape
+    if copies:
+        out = torch.empty((T, copies, E), dtype=torch.float32, device=table.device)
+        _check(_lib().illm_embed_streams(_p(tokens), _p(table), _code(table), _p(out), T, E, V,
+                                         int(copies), ctypes.c_float(scale), _stream()), "embed")
+        return out
     out = torch.empty((T, E), dtype=torch.float32, device=table.device)
     _check(_lib().illm_embed_scaled(_p(tokens), _p(table), _code(table), _p(out), T, E, V,
                                     ctypes.c_float(scale), _stream()), "embed")
@@ -117,6 +123,24 @@ def sum_rows(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     _check(_lib().illm_sum_rows(_p(a), _code(a), _p(b), _code(b), _p(out),
                                 ctypes.c_size_t(a.numel()), _stream()), "sum_rows")
     return out
+
+
+class ScaledSum:
+    """sa a + sb b of two parts' outputs for the same rows, not yet added: a block that can add it
+    in a kernel of its own takes the pieces, any other asks for `tensor()` (float32)."""
+
+    def __init__(self, a: torch.Tensor, sa: float, b: torch.Tensor, sb: float):
+        self.a, self.sa, self.b, self.sb = a, float(sa), b, float(sb)
+
+    def tensor(self) -> torch.Tensor:
+        a, b = self.a, self.b
+        _gpu(a, b)
+        _need(a.shape == b.shape, f"ScaledSum: {tuple(a.shape)} against {tuple(b.shape)}")
+        out = torch.empty(a.shape, dtype=torch.float32, device=a.device)
+        _check(_lib().illm_sum_rows_scaled(_p(a), _code(a), ctypes.c_float(self.sa), _p(b), _code(b),
+                                           ctypes.c_float(self.sb), _p(out),
+                                           ctypes.c_size_t(a.numel()), _stream()), "sum_rows_scaled")
+        return out
 
 
 def relu_squared(x: torch.Tensor) -> torch.Tensor:
@@ -161,6 +185,45 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         _p(weight), _code(weight),
         _p(out), _code(out), _p(row_idx), rows, E, ctypes.c_float(eps), _stream()), "add_rmsnorm")
     return out
+
+
+class StreamWrite:
+    """What a sublayer leaves for several residual streams: its output `y` (or `ya y + yb y2`, the
+    outputs of two parts that read the same rows) and how it enters them, x_t <- sum_s mix[s, t]
+    x_s + out[t] y (mix float32 [S, S] indexed [from, to], out float32 [S])."""
+
+    def __init__(self, y: torch.Tensor, mix: torch.Tensor, out: torch.Tensor,
+                 y2: Optional[torch.Tensor] = None, ya: float = 1.0, yb: float = 1.0):
+        self.y, self.mix, self.out, self.y2, self.ya, self.yb = y, mix, out, y2, float(ya), float(yb)
+
+
+def stream_mix_norm(x: torch.Tensor, write: Optional[StreamWrite], read: Optional[torch.Tensor],
+                    weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                    row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The write of one sublayer into the float32 residual streams x [T, S, E] (in place unless
+    `row_idx` picks rows) and the read and RMS norm of the next: u = sum_s read[s] x_s (no `read`:
+    the plain sum of the streams), rows u / sqrt(mean(u^2) + eps) * weight in `out_dtype`."""
+    _need(x.dtype == torch.float32 and x.dim() == 3, "stream_mix_norm: x must be float32 [T, S, E]")
+    T, S, E = x.shape
+    y = y2 = mix = out = None
+    ya = yb = 1.0
+    if write is not None:
+        y, y2, mix, out, ya, yb = write.y, write.y2, write.mix, write.out, write.ya, write.yb
+        _need(y.shape == (T, E) and (y2 is None or y2.shape == (T, E)), "stream_mix_norm: y must be [T, E]")
+        _need(mix.dtype == torch.float32 and mix.shape == (S, S) and out.dtype == torch.float32
+              and out.shape == (S,), "stream_mix_norm: mix float32 [S, S], out float32 [S]")
+    _gpu(x, y, y2, mix, out, read, weight, row_idx)
+    _i32(row_idx)
+    _need(read is None or (read.dtype == torch.float32 and read.shape == (S,)), "stream_mix_norm: read float32 [S]")
+    _need(weight.shape == (E,), f"stream_mix_norm: weight {tuple(weight.shape)} for width {E}")
+    rows = T if row_idx is None else row_idx.numel()
+    h = torch.empty((rows, E), dtype=out_dtype, device=x.device)
+    _check(_lib().illm_stream_mix_norm(
+        _p(x), S, _p(y), _code(y) if y is not None else 0, ctypes.c_float(ya), _p(y2),
+        _code(y2) if y2 is not None else 0, ctypes.c_float(yb), _p(mix), _p(out), _p(read), _p(weight),
+        _code(weight), _p(h), _code(h), _p(row_idx), rows, E, ctypes.c_float(eps), _stream()),
+        "stream_mix_norm")
+    return h
 
 
 def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
@@ -1229,9 +1292,15 @@ def few_outputs_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return z
 
 
-def moe_route(z: torch.Tensor, correction: Optional[torch.Tensor], top: int):
+MOE_SCORES = {"softmax": 0, "sigmoid": 1}            # a router's scores: over all outputs, or each its own
+MOE_ACTIVATIONS = {"silu": 0, "clamped_swish": 1}    # see `moe_experts`
+
+
+def moe_route(z: torch.Tensor, correction: Optional[torch.Tensor], top: int, score: str = "softmax"):
     """(idx int32 [T, top], weight float32 [T, top]): per row of the router's float32 outputs z
-    the `top` largest softmax(z) + correction, and their softmax values."""
+    the `top` largest score(z) + correction, and their scores (`score`: "softmax" over all
+    outputs, or "sigmoid" of each)."""
+    _need(score in MOE_SCORES, f"moe_route: score {score!r}; known: {sorted(MOE_SCORES)}")
     _gpu(z, correction)
     _need(z.dtype == torch.float32 and z.dim() == 2, "moe_route: float32 [T, outputs]")
     T, NE = z.shape
@@ -1240,7 +1309,7 @@ def moe_route(z: torch.Tensor, correction: Optional[torch.Tensor], top: int):
     wt = torch.empty((T, top), dtype=torch.float32, device=z.device)
     _check(_lib().illm_moe_route(_p(z), _p(correction),
                                  _code(correction) if correction is not None else 0, T, NE, top,
-                                 _p(idx), _p(wt), _stream()), "moe_route")
+                                 _p(idx), _p(wt), MOE_SCORES[score], _stream()), "moe_route")
     return idx, wt
 
 
@@ -1271,23 +1340,32 @@ def _moe_group(idx: torch.Tensor, n_exp: int, dtype: torch.dtype, E: int, F: int
 
 
 def moe_plan(h: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int,
-             w_gate_up: Optional[torch.Tensor]):
+             w_gate_up: Optional[torch.Tensor], score: str = "softmax"):
     """A routed layer's plan for the rows h: (idx, weight, grouped).  idx, weight [T, top] as
     `moe_route` gives them for the router's float32 outputs h . w_router^T; grouped: the pairs
     grouped by expert for `moe_experts` (None without stacked experts)."""
     E = h.shape[1]
     n_exp = w_gate_up.shape[0] if w_gate_up is not None else 0
-    idx, wt = moe_route(few_outputs_f32(h, w_router), correction, top)
+    idx, wt = moe_route(few_outputs_f32(h, w_router), correction, top, score)
     grouped = _moe_group(idx, n_exp, h.dtype, E, w_gate_up.shape[1] // 2) if n_exp else None
     return idx, wt, grouped
 
 
 def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
-                grouped=None) -> torch.Tensor:
+                grouped=None, activation: str = "silu", limit: float = 0.0,
+                input_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Y [T * top, E]: for every (token, choice) pair whose choice is one of the stacked experts
     (w_gate_up [experts, 2 F, E] = [gate | up], w_down [experts, E, F]) the expert's
-    down(silu(gate h) * (up h)); rows of other pairs are not written.  `grouped`: the pairs by
-    expert as `moe_plan` left them (else they are grouped here)."""
+    down(act(gate h, up h)); rows of other pairs are not written.  `activation` "silu":
+    silu(g) * u; "clamped_swish": with g = min(g, limit) and u = clamp(u, -limit, limit),
+    g * sigmoid(1.702 g) * (u + 1).  `input_weight` float32 [T, top]: the pair's expert sees
+    weight * h instead of h.  `grouped`: the pairs by expert as `moe_plan` left them (else they
+    are grouped here)."""
+    _need(activation in MOE_ACTIVATIONS, f"moe_experts: activation {activation!r}; known: {sorted(MOE_ACTIVATIONS)}")
+    act_kind, lim = MOE_ACTIVATIONS[activation], ctypes.c_float(limit)
+    _need(input_weight is None or (input_weight.dtype == torch.float32 and input_weight.numel() == idx.numel()),
+          "moe_experts: input weights are float32 [T, top]")
+    _gpu(input_weight)
     _gpu(h, idx, w_gate_up, w_down)
     _i32(idx)
     T, E = h.shape
@@ -1303,22 +1381,26 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gate_up: torch.Tensor, w_d
     y = torch.empty((NP, E), dtype=h.dtype, device=h.device)
     if mfma:
         _check(_lib().illm_moe_rows_mfma(_p(h), top, _p(w_gate_up), 1, rows, _p(order), _p(tiles),
-                                         max_tiles, _p(act), F, E, _stream()), "moe_rows_mfma (gate|up)")
+                                         max_tiles, _p(act), F, E, act_kind, lim, _p(input_weight),
+                                         _stream()), "moe_rows_mfma (gate|up)")
         _check(_lib().illm_moe_rows_mfma(_p(act), 1, _p(w_down), 0, rows, _p(order), _p(tiles),
-                                         max_tiles, _p(y), E, F, _stream()), "moe_rows_mfma (down)")
+                                         max_tiles, _p(y), E, F, 0, ctypes.c_float(0.0), _p(None),
+                                         _stream()), "moe_rows_mfma (down)")
         return y
     _check(_lib().illm_moe_rows(_p(h), top, _p(w_gate_up), _code(h), 1, _p(order), _p(tiles),
-                                max_tiles, _p(act), F, E, _stream()), "moe_rows (gate|up)")
+                                max_tiles, _p(act), F, E, act_kind, lim, _p(input_weight), _stream()),
+           "moe_rows (gate|up)")
     _check(_lib().illm_moe_rows(_p(act), 1, _p(w_down), _code(h), 0, _p(order), _p(tiles),
-                                max_tiles, _p(y), E, F, _stream()), "moe_rows (down)")
+                                max_tiles, _p(y), E, F, 0, ctypes.c_float(0.0), _p(None), _stream()),
+           "moe_rows (down)")
     return y
 
 
-def moe_combine(h: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor, y: Optional[torch.Tensor],
+def moe_combine(h: torch.Tensor, idx: torch.Tensor, wt: Optional[torch.Tensor], y: Optional[torch.Tensor],
                 n_real: int, shared: Optional[torch.Tensor] = None,
                 shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """float32 [T, E]: sum over a token's choices of weight * (the expert's row of y, or h itself
-    for a choice >= n_real), plus sigmoid(h . shared_gate) * shared."""
+    for a choice >= n_real), plus sigmoid(h . shared_gate) * shared.  `wt` None: every weight 1."""
     _gpu(h, idx, wt, y, shared, shared_gate)
     T, E = h.shape
     top = idx.shape[1]
@@ -1331,6 +1413,174 @@ def moe_combine(h: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor, y: Optiona
                                    _p(shared_gate),
                                    _code(shared_gate) if shared_gate is not None else 0, _p(out), T,
                                    E, top, n_real, _stream()), "moe_combine")
+    return out
+
+
+# ------------------------------------------------------------------ attention with a soft cap
+def kv_store2(rows: torch.Tensor, k_off: int, v_off: int, row_pos: torch.Tensor,
+              row_slot: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+              page_table: torch.Tensor, page_size: int, ring: int, nkv: int, dk: int, dv: int) -> None:
+    """Store the keys (columns k_off .. of width nkv dk) and values (v_off .. of width nkv dv) of
+    packed rows into the paged cache, K [pages, nkv, page_size, dk], V [pages, nkv, page_size, dv]."""
+    _gpu(rows, row_pos, row_slot, kcache, vcache, page_table)
+    T = rows.shape[0]
+    _i32(row_pos, T); _i32(row_slot, T); _i32(page_table)
+    _need(rows.dim() == 2 and kcache.dtype == rows.dtype and vcache.dtype == rows.dtype,
+          "kv_store2: rows [T, n] and a cache of their dtype")
+    _need(kcache.shape[1:] == (nkv, page_size, dk) and vcache.shape[1:] == (nkv, page_size, dv)
+          and kcache.shape[0] == vcache.shape[0] and page_table.dim() == 2, "kv_store2: cache shapes")
+    _check(_lib().illm_kv_store2(_p(rows), _code(rows), rows.shape[1], k_off, v_off, _p(row_pos),
+                                 _p(row_slot), _p(kcache), _p(vcache), _p(page_table),
+                                 page_table.shape[1], page_size, ring, T, nkv, dk, dv, _stream()),
+           "kv_store2")
+
+
+def _cap_cache_ok(q, kcache, vcache, page_table, page_size, nh, nkv, dk, dv, what):
+    _need(q.dim() == 2 and q.shape[1] >= nh * dk, f"{what}: rows [q | ...]")
+    _need(nh % nkv == 0, f"{what}: heads must be a multiple of kv heads")
+    _need(kcache.dtype == q.dtype and vcache.dtype == q.dtype
+          and kcache.shape[1:] == (nkv, page_size, dk) and vcache.shape[1:] == (nkv, page_size, dv)
+          and page_table.dim() == 2, f"{what}: cache shape or dtype")
+
+
+def attn_cap_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Tensor,
+                  seq_start: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                  page_table: torch.Tensor, page_size: int, ring: int, n_seqs: int, max_rows: int,
+                  nh: int, nkv: int, dk: int, dv: int, scale: float, cap: float,
+                  window: int) -> torch.Tensor:
+    """Causal attention of a step's packed rows over the paged cache (which holds the step's own
+    keys and values by now): row r of sequence b stands at position seq_start[b] + r; scores
+    cap tanh(q . k scale / cap) (cap 0: none); queries and keys of width dk, values of dv.
+    Returns [T, nh dv]."""
+    _gpu(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table)
+    _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs); _i32(seq_start, n_seqs); _i32(page_table)
+    _cap_cache_ok(q, kcache, vcache, page_table, page_size, nh, nkv, dk, dv, "attn_cap_rows")
+    out = torch.empty((q.shape[0], nh * dv), dtype=q.dtype, device=q.device)
+    if (q.dtype == torch.bfloat16 and attn_cap_mfma_fits(dk, dv, page_size)):
+        _check(_lib().illm_attn_cap_rows_bf16(
+            _p(q), q.shape[1], _p(out), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
+            _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_rows, nh,
+            nkv, dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _stream()),
+            f"attn_cap_rows_bf16 (sizes {dk}, {dv})")
+        return out
+    _check(_lib().illm_attn_cap_rows(
+        _p(q), q.shape[1], _p(out), _code(q), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
+        _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_rows, nh, nkv,
+        dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _stream()),
+        f"attn_cap_rows (sizes {dk}, {dv})")
+    return out
+
+
+ATTN_CAP_MFMA = False
+
+
+def attn_cap_mfma_fits(dk: int, dv: int, page_size: int) -> bool:
+    return ATTN_CAP_MFMA and dk % 16 == 0 and dv % 16 == 0 and page_size % 64 == 0
+
+
+def attn_cap_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                    page_table: torch.Tensor, page_size: int, ring: int, seq_slot: torch.Tensor,
+                    seq_len: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, scale: float,
+                    cap: float, window: int, nsplit: int) -> torch.Tensor:
+    """The same attention for one new token per sequence: row b of q against the seq_len[b] keys
+    (the new one included) of its slot, the keys cut into `nsplit` ranges.  Returns [B, nh dv]."""
+    _gpu(q, kcache, vcache, page_table, seq_slot, seq_len)
+    B = q.shape[0]
+    _i32(page_table); _i32(seq_slot, B); _i32(seq_len, B)
+    _cap_cache_ok(q, kcache, vcache, page_table, page_size, nh, nkv, dk, dv, "attn_cap_decode")
+    out = torch.empty((B, nh * dv), dtype=q.dtype, device=q.device)
+    partial = torch.empty((B, nh, nsplit, dv + 2), dtype=torch.float32, device=q.device)
+    _check(_lib().illm_attn_cap_decode(
+        _p(q), q.shape[1], _p(out), _code(q), _p(kcache), _p(vcache), _p(page_table),
+        page_table.shape[1], page_size, ring, _p(seq_slot), _p(seq_len), _p(partial), nsplit, B, nh,
+        nkv, dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _stream()),
+        f"attn_cap_decode (sizes {dk}, {dv})")
+    return out
+
+
+# ------------------------------------------------------------------ the gated delta rule
+def delta_prepare(P: torch.Tensor, b_off: int, A: torch.Tensor, a_off: int, conv_w: torch.Tensor,
+                  tail: torch.Tensor, row_slot: torch.Tensor, a_log: torch.Tensor,
+                  dt_bias: torch.Tensor, G: int, H: int, dk: int, dv: int, per_channel: bool):
+    """From the projections P [T, n] = [q (G dk) | k (G dk) | v (H dv) | ...] the recurrence's
+    float32 inputs: q and k after the short convolution (conv_w float32 [C, taps], the inputs
+    before a step's first row from `tail` [slots, taps - 1, C]), SiLU and the unit norm per head
+    (q also times dk^-1/2), v after convolution and SiLU, beta = sigmoid(P[:, b_off + h]) and the
+    decays exp(-exp(a_log[h]) softplus(A[:, a_off + i] + dt_bias[i])), one a head or, with
+    `per_channel`, one a head and key channel.  Returns (q [T, G, dk], k, v [T, H, dv],
+    beta [T, H], decay [T, H, 1 or dk])."""
+    _gpu(P, A, conv_w, tail, row_slot, a_log, dt_bias)
+    T = P.shape[0]
+    _i32(row_slot, T)
+    C = 2 * G * dk + H * dv
+    DW = dk if per_channel else 1
+    _need(P.dim() == 2 and P.shape[1] >= max(C, b_off + H) and A.dim() == 2 and A.shape[0] == T
+          and A.shape[1] >= a_off + H * DW, "delta_prepare: projections too narrow")
+    _need(conv_w.dtype == torch.float32 and conv_w.dim() == 2 and conv_w.shape[0] == C,
+          "delta_prepare: conv_w float32 [C, taps]")
+    taps = conv_w.shape[1]
+    _need(tail.dim() == 3 and tail.shape[1:] == (max(taps - 1, 1), C), "delta_prepare: tail [slots, taps - 1, C]")
+    _need(a_log.dtype == torch.float32 and a_log.shape == (H,) and dt_bias.dtype == torch.float32
+          and dt_bias.numel() == H * DW, "delta_prepare: a_log float32 [H], dt_bias float32 [H (dk)]")
+    dev = P.device
+    qn = torch.empty((T, G, dk), dtype=torch.float32, device=dev)
+    kn = torch.empty((T, G, dk), dtype=torch.float32, device=dev)
+    vv = torch.empty((T, H, dv), dtype=torch.float32, device=dev)
+    beta = torch.empty((T, H), dtype=torch.float32, device=dev)
+    dec = torch.empty((T, H, DW), dtype=torch.float32, device=dev)
+    _check(_lib().illm_delta_prepare(
+        _p(P), _code(P), P.shape[1], b_off, _p(A), _code(A), A.shape[1], a_off, _p(conv_w), taps,
+        _p(tail), _code(tail), _p(row_slot), _p(a_log), _p(dt_bias), _p(qn), _p(kn), _p(vv), _p(beta),
+        _p(dec), T, G, H, dk, dv, DW, _stream()), "delta_prepare")
+    return qn, kn, vv, beta, dec
+
+
+def delta_conv_tail(P: torch.Tensor, tail: torch.Tensor, cu_seqlens: torch.Tensor,
+                    seq_slot: torch.Tensor, n_seqs: int, taps: int) -> None:
+    """Keep the last taps - 1 convolution inputs of every sequence of the step in `tail`."""
+    _gpu(P, tail, cu_seqlens, seq_slot)
+    _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs)
+    C = tail.shape[2]
+    _need(P.dim() == 2 and P.shape[1] >= C and tail.shape[1] == max(taps - 1, 1), "delta_conv_tail: shapes")
+    _check(_lib().illm_delta_conv_tail(_p(P), _code(P), P.shape[1], _p(tail), _code(tail),
+                                       _p(cu_seqlens), _p(seq_slot), n_seqs, C, taps, _stream()),
+           "delta_conv_tail")
+
+
+def delta_scan(qn, kn, vv, beta, dec, state: torch.Tensor, cu_seqlens: torch.Tensor,
+               seq_slot: torch.Tensor, n_seqs: int) -> torch.Tensor:
+    """The recurrence S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q over every
+    sequence's rows in order, from `state` float32 [slots, H, dk, dv] and back into it.
+    Returns o float32 [T, H, dv]."""
+    _gpu(qn, kn, vv, beta, dec, state, cu_seqlens, seq_slot)
+    _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs)
+    T, G, dk = qn.shape
+    _, H, dv = vv.shape
+    _need(all(t.dtype == torch.float32 for t in (qn, kn, vv, beta, dec, state)), "delta_scan: float32")
+    _need(kn.shape == qn.shape and beta.shape == (T, H) and dec.shape[:2] == (T, H)
+          and dec.shape[2] in (1, dk) and state.shape[1:] == (H, dk, dv), "delta_scan: shapes")
+    o = torch.empty((T, H, dv), dtype=torch.float32, device=qn.device)
+    _check(_lib().illm_delta_scan(_p(qn), _p(kn), _p(vv), _p(beta), _p(dec), dec.shape[2], _p(state),
+                                  _p(cu_seqlens), _p(seq_slot), _p(o), n_seqs, G, H, dk, dv, _stream()),
+           "delta_scan")
+    return o
+
+
+DELTA_GATES = {"silu": 0, "sigmoid": 1}
+
+
+def delta_finish(o: torch.Tensor, weight: torch.Tensor, Z: torch.Tensor, z_off: int, gate: str,
+                 eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """[T, H dv] rows o / sqrt(mean over dv of o^2 + eps) * weight [dv] * act(Z[:, z_off + ...]),
+    act "silu" or "sigmoid", per head."""
+    _gpu(o, weight, Z)
+    T, H, dv = o.shape
+    _need(o.dtype == torch.float32 and weight.shape == (dv,) and Z.dim() == 2 and Z.shape[0] == T
+          and Z.shape[1] >= z_off + H * dv and gate in DELTA_GATES, "delta_finish: shapes or gate")
+    out = torch.empty((T, H * dv), dtype=out_dtype, device=o.device)
+    _check(_lib().illm_delta_finish(_p(o), _p(weight), _code(weight), _p(Z), _code(Z), Z.shape[1], z_off,
+                                    DELTA_GATES[gate], _p(out), _code(out), T, H, dv,
+                                    ctypes.c_float(eps), _stream()), "delta_finish")
     return out
 
 

@@ -1,3 +1,3 @@
-from . import llama, rabapel  # registers LlamaForCausalLM and Rabapel
+from . import kukupel, llama, rabapel  # registers Kukupel, LlamaForCausalLM and Rabapel
 
-__all__ = ["llama", "rabapel"]
+__all__ = ["kukupel", "llama", "rabapel"]

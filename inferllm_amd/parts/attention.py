@@ -129,3 +129,77 @@ class Attention(Mixer):
                                   next_norm.rms_params() if next_norm is not None else None,
                                   ctx.act_dtype)
         return ops.linear(o, self.w_o)
+
+
+@register_part("mixer", "capped_attention")
+class CappedAttention(Mixer):
+    """Causal attention with grouped kv heads, a soft cap on the scores and value heads of a width
+    of their own, without a position encoding:
+
+        score = softcap * tanh((q . k) * softmax_scale / softcap)      (softcap 0: no cap)
+
+    then the softmax over the visible keys (every j <= i, or the last `window`) and the sum of the
+    values.  Queries and keys have `key_dim` dims a head, values `value_dim`; query head h reads
+    kv head h / (num_heads / num_kv_heads).  A step stores its keys and values in the paged cache
+    first and every row attends over the cache at its position, so prompts, portions of prompts
+    and single tokens run the same way.
+    """
+
+    graph_safe_prompts = True
+    takes_continuations = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int,
+                 value_dim: int, softmax_scale: Optional[float] = None, softcap: float = 0.0,
+                 window: Optional[int] = None, tensors=None):
+        super().__init__(tensors)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if key_dim > 256 or value_dim > 256:
+            raise ValueError(f"head sizes {key_dim}, {value_dim} are beyond the attention kernels' limit of 256")
+        self.E, self.nh, self.nkv = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.dk, self.dv = int(key_dim), int(value_dim)
+        self.window = int(window) if window else None
+        self.scale = float(softmax_scale) if softmax_scale else 1.0 / math.sqrt(self.dk)
+        self.softcap = float(softcap or 0.0)
+        self.w_qkv = self.w_o = None
+
+    def shapes(self) -> Dict[str, TensorWant]:
+        return {"q": TensorWant((self.nh * self.dk, self.E)),
+                "k": TensorWant((self.nkv * self.dk, self.E)),
+                "v": TensorWant((self.nkv * self.dv, self.E)),
+                "o": TensorWant((self.E, self.nh * self.dv))}
+
+    def kv_spec(self) -> KVSpec:
+        from ..cache.manager import TokenTensor
+        return KVSpec("window" if self.window else "full",
+                      (TokenTensor("k", (self.nkv, self.dk)), TokenTensor("v", (self.nkv, self.dv))),
+                      self.window)
+
+    def load(self, tensors) -> None:
+        self.w_qkv = ops.decode_weight(_fuse([self._take(tensors, n) for n in ("q", "k", "v")]),
+                                       "plain", self.decode_copies)
+        self.w_o = ops.decode_weight(self._take(tensors, "o").contiguous(), "plain", self.decode_copies)
+
+    def tunables(self):
+        return (("plain", self.w_o, {}),)
+
+    def forward(self, h, ctx: StepContext, line, writes_cache, position):
+        nh, nkv, dk, dv = self.nh, self.nkv, self.dk, self.dv
+        kc, vc, group = ctx.cache.kv_line(line)
+        window = self.window or 0
+        qkv = ops.linear(h, self.w_qkv)
+        if writes_cache:
+            ops.kv_store2(qkv, nh * dk, (nh + nkv) * dk, ctx.row_pos, ctx.row_slot, kc, vc, group.table,
+                          group.page_size, group.ring, nkv, dk, dv)
+        if ctx.prefill:
+            o = ops.attn_cap_rows(qkv, ctx.cu_seqlens, ctx.seq_slot, ctx.seq_start, kc, vc, group.table,
+                                  group.page_size, group.ring, ctx.n_seqs, ctx.max_rows, nh, nkv, dk,
+                                  dv, self.scale, self.softcap, window)
+        else:
+            longest = min(ctx.max_len, window) if window else ctx.max_len
+            tiles = max(1, (longest + 63) // 64)
+            nsplit = max(1, min(-(-512 // max(1, ctx.n_seqs * nh)), 16, tiles))
+            o = ops.attn_cap_decode(qkv, kc, vc, group.table, group.page_size, group.ring,
+                                    ctx.seq_slot, ctx.seq_len, nh, nkv, dk, dv, self.scale,
+                                    self.softcap, window, nsplit)
+        return ops.linear(o, self.w_o)

@@ -122,8 +122,9 @@ class Mixer(Part):
         """Keys/values the mixer keeps per token, or None."""
         return None
 
-    def state_spec(self) -> Optional[StateSpec]:
-        """Fixed-size state the mixer keeps per sequence, or None."""
+    def state_spec(self):
+        """Fixed-size state the mixer keeps per sequence: a `StateSpec`, a dict name -> StateSpec
+        if it keeps several tensors, or None."""
         return None
 
     def forward(self, h: torch.Tensor, ctx: StepContext, line: int, writes_cache: bool,
@@ -189,8 +190,9 @@ class Block(Part):
     takes_prepared_rows = False
 
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
-                 feed_forward_norm: Optional[Norm], position: Optional[PositionEncoding]):
-        super().__init__()
+                 feed_forward_norm: Optional[Norm], position: Optional[PositionEncoding],
+                 tensors: Optional[Dict[str, str]] = None):
+        super().__init__(tensors)
         self.mixer, self.feed_forward = mixer, feed_forward
         self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
         self.position = position
@@ -201,13 +203,17 @@ class Block(Part):
         return ps
 
     def wants(self) -> Dict[str, TensorWant]:
-        out: Dict[str, TensorWant] = {}
+        out: Dict[str, TensorWant] = dict(super().wants())       # the arrangement's own tensors
         for p in self.parts():
             out.update(p.wants())
         return out
 
+    def load_own(self, tensors) -> None:
+        """Take the arrangement's own tensors (those of `shapes()`); most have none."""
+
     def load(self, tensors) -> None:
         self.mixer.position = self.position      # a mixer may lay its matrices out for the encoding
+        self.load_own(tensors)
         for p in self.parts():
             p.load(tensors)
 

@@ -1,7 +1,10 @@
 """Arrangements of mixer, feed-forward and norms around the residual stream."""
 from __future__ import annotations
 
+import torch
+
 from ..kernels import ops
+from ..weights.loader import TensorWant
 from .base import Block, StepContext, register_part
 
 
@@ -74,3 +77,53 @@ class ParallelBlock(Block):
         if next_norm is not None and getattr(next_norm, "adds_pairs", False):
             return (a, f)
         return ops.sum_rows(a, f)
+
+
+@register_part("block", "hyper_connections")
+class HyperConnectionBlock(Block):
+    """Pre-norm sublayers over `streams` residual streams x_1 .. x_s in place of one.
+
+    For each sublayer q (the mixer, then the feed-forward): u = sum_s read_q[s] x_s,
+    y = sublayer(norm_q(u)), then for all streams at once x_t <- sum_s mix_q[s, t] x_s + out_q[t] y.
+    The reads belong to the norms (`stream_rms_norm`, whose kernel also does the write of the
+    sublayer before it); the block owns mix_q [streams, streams] (indexed [from, to]) and out_q
+    [streams] and hands each sublayer's output on as `ops.StreamWrite`, the last one to whatever
+    norm comes next.  A layer whose feed-forward is "none" has the mixer's sublayer alone.
+    """
+
+    graph_safe_prompts = True
+
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm, position, streams: int,
+                 tensors=None):
+        super().__init__(mixer, feed_forward, mixer_norm, feed_forward_norm, position, tensors)
+        self.streams = int(streams)
+        self.has_ff = feed_forward_norm is not None
+        if hasattr(mixer, "takes_scaled_sums"):
+            mixer.takes_scaled_sums = True       # the streams' kernel adds sa a + sb b itself
+        self.mix = [None, None]
+        self.out = [None, None]
+
+    def shapes(self):
+        S = self.streams
+        mix = lambda: TensorWant((S, S), init="eye_normal", keep_stored=True)
+        out = lambda: TensorWant((S,), init="ones_normal", keep_stored=True)
+        out = {"mix1": mix(), "out1": out()} | ({"mix2": mix(), "out2": out()} if self.has_ff else {})
+        return out
+
+    def load_own(self, tensors) -> None:
+        for q in range(2 if self.has_ff else 1):
+            self.mix[q] = self._take(tensors, f"mix{q + 1}").to(torch.float32).contiguous()
+            self.out[q] = self._take(tensors, f"out{q + 1}").to(torch.float32).contiguous()
+
+    def _write(self, y, q: int) -> ops.StreamWrite:
+        if isinstance(y, ops.ScaledSum):
+            return ops.StreamWrite(y.a, self.mix[q], self.out[q], y2=y.b, ya=y.sa, yb=y.sb)
+        return ops.StreamWrite(y, self.mix[q], self.out[q])
+
+    def forward(self, x, pending, ctx: StepContext, line, writes_cache):
+        h = self.mixer_norm.forward(x, pending, ctx)
+        first = self._write(self.mixer.forward(h, ctx, line, writes_cache, self.position), 0)
+        if not self.has_ff:
+            return first
+        h2 = self.feed_forward_norm.forward(x, first, ctx)
+        return self._write(self.feed_forward.forward(h2, ctx), 1)

@@ -13,14 +13,16 @@ from .base import Embedding, Head, StepContext, register_part
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Embedding):
     """Row copy (src/kern/naive/naive.cpp:43-54); rows become float32 and are multiplied by
-    `scale` (1: the reference's plain copy)."""
+    `scale` (1: the reference's plain copy).  `streams` > 0: a model with several residual
+    streams; the rows come out as [rows, streams, hidden], every stream the embedded row."""
 
     graph_safe_prompts = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, tensors=None):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, streams: int = 0,
+                 tensors=None):
         super().__init__(tensors)
         self.V, self.E = int(vocab_size), int(hidden_size)
-        self.scale = float(scale)
+        self.scale, self.streams = float(scale), int(streams)
         self.weight: Optional[torch.Tensor] = None
 
     def shapes(self) -> Dict[str, TensorWant]:
@@ -30,7 +32,7 @@ class TokenEmbedding(Embedding):
         self.weight = self._take(tensors, "weight").contiguous()
 
     def forward(self, ctx: StepContext):
-        return ops.embed(ctx.tokens, self.weight, self.scale)
+        return ops.embed(ctx.tokens, self.weight, self.scale, self.streams)
 
 
 @register_part("head", "lm_head")

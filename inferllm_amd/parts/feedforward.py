@@ -115,6 +115,10 @@ class RoutedExperts(FeedForward):
 
     The weights are the chosen scores as they are (no renormalisation).  `shared_size` > 0 adds
     an expert that every token uses, scaled per token by a sigmoid gate if `shared_gate`.
+    `score` "sigmoid" scores every router output by its own sigmoid instead of the softmax over
+    all.  `activation` "clamped_swish" with `limit`: g = min(W_gate h, limit), u = clamp(W_up h,
+    -limit, limit), expert(h) = W_down (g sigmoid(1.702 g) (u + 1)).  `weight_on` "input": the
+    weight multiplies what the expert reads, out = sum over chosen e of expert_e(s_e h).
     Tensor parameters: "router", "correction", "e<i>.gate" / ".up" / ".down", "shared.gate" /
     ".up" / ".down", "shared.sg".  The result is float32.
     """
@@ -123,8 +127,19 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, hidden_size: int, expert_size: int, num_experts: int, top: int,
                  num_identity: int = 0, correction: bool = True, shared_size: int = 0,
-                 shared_gate: bool = True, tensors=None):
+                 shared_gate: bool = True, score: str = "softmax", activation: str = "silu",
+                 limit: float = 0.0, weight_on: str = "output", tensors=None):
         super().__init__(tensors)
+        if score not in ops.MOE_SCORES or activation not in ops.MOE_ACTIVATIONS:
+            raise ValueError(f"routed experts: score {score!r} or activation {activation!r} is unknown; "
+                             f"known: {sorted(ops.MOE_SCORES)}, {sorted(ops.MOE_ACTIVATIONS)}")
+        if weight_on not in ("output", "input"):
+            raise ValueError(f"routed experts: weight_on {weight_on!r} is neither 'output' nor 'input'")
+        if activation == "clamped_swish" and not float(limit) > 0:
+            raise ValueError("routed experts: the clamped activation needs a positive limit")
+        if weight_on == "input" and int(num_identity):
+            raise ValueError("routed experts: identity experts take their weight on the output")
+        self.score, self.activation, self.limit, self.weight_on = score, activation, float(limit), weight_on
         self.E, self.F = int(hidden_size), int(expert_size)
         self.n_real, self.n_id, self.top = int(num_experts), int(num_identity), int(top)
         self.has_correction, self.Fs = bool(correction), int(shared_size)
@@ -172,8 +187,13 @@ class RoutedExperts(FeedForward):
                 self.w_sg = take("shared.sg").reshape(-1).contiguous()
 
     def forward(self, h, ctx: StepContext):
-        idx, weight, grouped = ops.moe_plan(h, self.w_router, self.correction, self.top, self.w_gate_up)
-        y = ops.moe_experts(h, idx, self.w_gate_up, self.w_down, grouped) if self.n_real else None
+        idx, weight, grouped = ops.moe_plan(h, self.w_router, self.correction, self.top,
+                                            self.w_gate_up, self.score)
+        on_input = self.weight_on == "input"
+        y = (ops.moe_experts(h, idx, self.w_gate_up, self.w_down, grouped, self.activation, self.limit,
+                             weight if on_input else None) if self.n_real else None)
+        if on_input:
+            weight = None                        # the experts' rows are summed as they are
         shared = None
         if self.Fs:
             shared = ops.linear(ops.gate_up_silu(h, self.w_shared_gate_up), self.w_shared_down)

@@ -41,3 +41,39 @@ class RMSNorm(Norm):
 
     def forward(self, x, delta, ctx: StepContext, row_idx=None):
         return ops.add_rmsnorm(x, delta, self.weight, self.eps, ctx.act_dtype, row_idx)
+
+
+@register_part("norm", "stream_rms_norm")
+class StreamRMSNorm(Norm):
+    """The norm in front of a sublayer of a model with several residual streams: the write of the
+    sublayer before (`ops.StreamWrite`: x_t <- sum_s mix[s, t] x_s + out[t] y for all streams at
+    once), the read u = sum_s read[s] x_s and y = u / sqrt(mean(u^2) + eps) * weight, in one kernel.
+    x is float32 [rows, streams, size].  Without a `read` tensor the streams are summed as they
+    are (the model's last norm)."""
+
+    graph_safe_prompts = True
+
+    def __init__(self, size: int, eps: float, streams: int, tensors=None):
+        super().__init__(tensors)
+        self.size, self.eps, self.streams = int(size), float(eps), int(streams)
+        if not 1 <= self.streams <= 8:
+            raise ValueError(f"{streams} residual streams: the kernels take 1 to 8")
+        self.weight: Optional[torch.Tensor] = None
+        self.read: Optional[torch.Tensor] = None
+
+    def shapes(self) -> Dict[str, TensorWant]:
+        out = {"weight": TensorWant((self.size,), init="ones_normal", keep_stored=True)}
+        if "read" in self.tensors:
+            out["read"] = TensorWant((self.streams,), init="ones_normal", keep_stored=True)
+        return out
+
+    def load(self, tensors) -> None:
+        self.weight = self._take(tensors, "weight").contiguous()
+        if "read" in self.tensors:
+            self.read = self._take(tensors, "read").to(torch.float32).contiguous()
+
+    def forward(self, x, delta, ctx: StepContext, row_idx=None):
+        if delta is not None and not isinstance(delta, ops.StreamWrite):
+            raise TypeError("stream_rms_norm adds what a block of several streams leaves "
+                            "(ops.StreamWrite), not plain rows")
+        return ops.stream_mix_norm(x, delta, self.read, self.weight, self.eps, ctx.act_dtype, row_idx)

@@ -55,7 +55,8 @@ class TensorWant:
     """What the model needs of one checkpoint tensor."""
     shape: Tuple[int, ...]
     kind: str = "float"          # "float" or "int"
-    init: str = "normal"         # random-weights rule: "normal" N(0, s) or "ones_normal" 1 + N(0, s)
+    init: str = "normal"         # random-weights rule: "normal" N(0, s), "ones_normal" 1 + N(0, s),
+                                 # "eye_normal" identity + N(0, s)
     optional: bool = False       # absent is fine (e.g. a head tied to the embedding)
     keep_stored: bool = False    # keeps the file's precision in a bfloat16 engine (norm weights)
 
@@ -93,6 +94,16 @@ def kept_dtype(stored: torch.dtype, kind: str, engine_dtype: torch.dtype,
     if stored == torch.bfloat16 or not keep_stored:
         return torch.bfloat16
     return torch.float32
+
+
+def stored_shapes(model_dir: str) -> Dict[str, Tuple[int, ...]]:
+    """Tensor name -> shape of everything the folder's safetensors files hold (headers only)."""
+    files: List[SafetensorsFile] = open_model_files(model_dir)
+    try:
+        return {n: tuple(e[1]) for f in files for n, e in f.entries.items()}
+    finally:
+        for f in files:
+            f.close()
 
 
 def load_named_tensors(model_dir: str, expected: Dict[str, TensorWant], engine_dtype: torch.dtype,

@@ -39,6 +39,8 @@ def random_tensor(seed: int, name: str, want: TensorWant, dtype: torch.dtype,
     t = torch.randn(want.shape, generator=g, dtype=torch.float32, device=device)
     if want.init == "ones_normal":
         t.mul_(NORM_STD).add_(1.0)
+    elif want.init == "eye_normal":          # a square mixing matrix: the identity + N(0, s)
+        t.mul_(NORM_STD).add_(torch.eye(want.shape[0], want.shape[1], dtype=torch.float32, device=device))
     elif want.init == "normal":
         t.mul_(LINEAR_STD)
     else:
