@@ -22,7 +22,8 @@ of MI355X (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, float32 157.3 TFLOP/s).
 The run fails (non-zero) if any timed run produced a non-finite logit or the same
 greedy token everywhere.
 
-`--design rabapel` is another workload with a line of its own (the default's stays as it is):
+`--design rabapel` and `--design kukupel` are other workloads with a line of their own (the
+default's stays as it is):
 Rabapel (latent attention, layers that alternate a dense and a routed feed-forward) at two
 sizes beside LLaMA at the same width, heads and layer count: prefill of 2,048 tokens and decoding
 at batch 1, 8 and 64, each with its fraction of the matrix or HBM peak.
@@ -318,6 +319,111 @@ def rabapel_main(args) -> int:
     return 0
 
 
+# ---------------------------------------------------------------- Kukupel beside Rabapel
+def kukupel_config(width, heads, kv_heads, layers, experts, expert_ff, top, streams=4, vocab=32000):
+    """Layers in the order parallel, parallel, delta, parallel ...: attention heads of 128 query
+    and 128 value dims beside delta-rule heads of 128 x 128 (a decay a key channel, low ranks of
+    64), delta-rule layers of the same heads alone, a routed feed-forward in every layer."""
+    delta = {"heads": heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4}
+    par = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                    "softcap": 30.0},
+           "right": dict(delta, decay_rank=64, gate_rank=64), "left_scale": 1.0, "right_scale": 1.0}
+    mlp = {"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0}, "router": {"experts": experts, "top": top}}
+    return {"architecture": "Kukupel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "streams": streams, "max_positions": 8192,
+            "layers": [{"type": "delta", "mixer": dict(delta), "mlp": mlp} if i % 4 == 2 else
+                       {"type": "parallel", "mixer": dict(par), "mlp": mlp} for i in range(layers)]}
+
+
+def kukupel_counts(cfg, esz):
+    """(step_bytes(batch, mean_ctx), flops(tokens, lens)) of a Kukupel configuration: the weights
+    a decode step reads (of a routed layer the router and the experts that `batch` tokens are
+    expected to choose), attention's cache rows and the delta rule's float32 states (read and
+    written); the multiply-adds of a prompt step (the recurrence as 3 key x value products a
+    token and head)."""
+    E, V = cfg["width"], cfg["vocab"]
+
+    def delta_parts(m, low):
+        H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        w = E * (2 * G * dk + H * dv + H) + E * H * dv
+        w += (E * (m["decay_rank"] + m["gate_rank"]) + m["decay_rank"] * H * dk + m["gate_rank"] * H * dv
+              if low else E * (H + H * dv))
+        return w, H * dk * dv
+
+    def layer_parts(layer):
+        m = layer["mixer"]
+        if layer["type"] == "delta":
+            w, state = delta_parts(m, False)
+            return w, state, 0, 0
+        l = m["left"]
+        w, state = delta_parts(m["right"], True)
+        w += E * (l["heads"] * l["dim"] + l["kv_heads"] * (l["dim"] + l["vdim"])) + E * l["heads"] * l["vdim"]
+        return w, state, l["kv_heads"] * (l["dim"] + l["vdim"]), l["heads"] * (l["dim"] + l["vdim"])
+
+    def step_bytes(batch, mean_ctx):
+        total = V * E * esz
+        for layer in cfg["layers"]:
+            w, state, kv_row, _ = layer_parts(layer)
+            r, ff = layer["mlp"]["router"], layer["mlp"]["expert"]["ff"]
+            used = r["experts"] * (1.0 - (1.0 - r["top"] / r["experts"]) ** batch)
+            total += (w + used * 3 * E * ff + batch * mean_ctx * kv_row) * esz + E * r["experts"] * 4
+            total += batch * state * 4 * 2
+        return total
+
+    def flops(tokens, lens):
+        total = 2.0 * len(lens) * V * E
+        pairs = sum(n * (n + 1) / 2 for n in lens)
+        for layer in cfg["layers"]:
+            w, state, _, qk = layer_parts(layer)
+            r, ff = layer["mlp"]["router"], layer["mlp"]["expert"]["ff"]
+            total += 2.0 * tokens * (w + E * r["experts"] + r["top"] * 3 * E * ff) + 2.0 * qk * pairs
+            total += 2.0 * 3 * state * tokens
+        return total
+
+    return step_bytes, flops
+
+
+def kukupel_main(args) -> int:
+    """Kukupel at two sizes beside Rabapel, the library's other design with routed feed-forwards,
+    at the same width, heads, experts and number of layers (four): tokens/s of these four-layer
+    models, with the fraction of the matrix peak for prompts and of the HBM peak for decode steps."""
+    import torch
+    from inferllm_amd import Engine
+    layers = args.layers or 4
+    esz = 2 if args.dtype == "bfloat16" else 4
+    sizes = {"2048": dict(width=2048, heads=16, kv_heads=4, experts=64, expert_ff=1408, top=6),
+             "4096": dict(width=4096, heads=32, kv_heads=8, experts=32, expert_ff=2048, top=4)}
+    few = min(args.steps, 128)
+    out = {"metric": "Kukupel beside Rabapel at equal width, heads, experts and layers: prefill tok/s at 2,048 tokens, decode tok/s at batch 1/8/64",
+           "unit": "tokens/s", "n_gpus": 1, "steps": few, "warmup": 4, "dtype": "bf16" if esz == 2 else "fp32",
+           "data": "synthetic: seeded random weights, uniform random token ids", "layers": layers, "sizes": {}}
+    for name, sz in sizes.items():
+        if args.size and args.size != name:
+            continue
+        row = {}
+        kcfg = kukupel_config(layers=layers, **sz)
+        rcfg = rabapel_config(width=sz["width"], heads=sz["heads"], layers=layers, dense_ff=4 * sz["width"],
+                              experts=sz["experts"], expert_ff=sz["expert_ff"], top=sz["top"],
+                              shared_ff=2 * sz["expert_ff"])
+        for design, cfg, counts in (("kukupel", kcfg, kukupel_counts), ("rabapel", rcfg, rabapel_counts)):
+            if args.only and args.only != design:
+                continue
+            eng = Engine.from_random(cfg, seed=0, dtype=args.dtype, device="cuda:0", max_batch=64,
+                                     max_seq_len=4096, max_tokens=64 * 1024)
+            b = Bench.around(eng, cfg["vocab"], layers, args.dtype, *counts(cfg, esz))
+            torch.cuda.synchronize()
+            r = {"prefill_2048": b.prefill_run(2048, reps=4)}
+            for batch in (1, 8, 64):
+                v, ms, f = b.decode_run(batch, few, 4, args.prompt)
+                r[f"decode_b{batch}"] = {"value": round(v, 1), "ms": round(ms, 4), "hbm_frac": round(f, 4)}
+            row[design] = r
+            b.close()
+            del b, eng
+        out["sizes"][name] = row
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -335,9 +441,11 @@ def main() -> int:
     ap.add_argument("--no-70b", action="store_true",
                     help="leave the LLaMA-2-70B shape out of `points` (138 GB of weights: half a minute)")
     ap.add_argument("--with-70b", action="store_true", help="(the default now; kept for old command lines)")
-    ap.add_argument("--design", default="llama", choices=["llama", "rabapel"],
-                    help="rabapel: that design at two sizes beside LLaMA at equal size (a line of its own)")
-    ap.add_argument("--size", default="", help="with --design rabapel: only this width (2048 or 4096)")
+    ap.add_argument("--design", default="llama", choices=["llama", "rabapel", "kukupel"],
+                    help="rabapel: that design at two sizes beside LLaMA at equal size (a line of its own); "
+                         "kukupel: that design at two sizes beside Rabapel at equal size (likewise)")
+    ap.add_argument("--size", default="", help="with --design rabapel or kukupel: only this width (2048 or 4096)")
+    ap.add_argument("--only", default="", help="with --design kukupel: only this one of the two designs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only (this library has no multi-GPU path); --gpus must be 1")
@@ -345,6 +453,8 @@ def main() -> int:
 
     if args.design == "rabapel":
         return rabapel_main(args)
+    if args.design == "kukupel":
+        return kukupel_main(args)
 
     shape_name, shape_cfg = SHAPES[args.shape]
     ctx_len = shape_cfg["max_position_embeddings"]

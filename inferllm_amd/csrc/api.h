@@ -87,6 +87,10 @@ int illm_attn_prefill_generic(const void* qkv, void* out, int dt, const int32_t*
 int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t* cu_seqlens, int n_seqs,
                            int max_len, int nh, int nkv, int hd, float scale, int window,
                            void* stream);
+// The same with a soft cap on the scores, cap tanh(score / cap) (cap <= 0: none).
+int illm_attn_prefill_bf16_cap(const void* qkv, void* out, const int32_t* cu_seqlens, int n_seqs,
+                           int max_len, int nh, int nkv, int hd, float scale, float cap, int window,
+                           void* stream);
 
 // The two above for steps whose rows go on from tokens the cache already holds (a prompt cut into
 // several steps): keys and values are read from the paged cache, which must hold the step's own
@@ -104,6 +108,12 @@ int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const int32_t* cu_s
                                  const void* kcache, const void* vcache, const int32_t* page_table,
                                  int table_stride, int page_size, int ring, int n_seqs, int max_len,
                                  int nh, int nkv, int hd, float scale, int window, void* stream);
+// The same with a soft cap on the scores, cap tanh(score / cap) (cap <= 0: none).
+int illm_attn_prefill_paged_bf16_cap(const void* qkv, void* out, const int32_t* cu_seqlens,
+                                 const int32_t* seq_slot, const int32_t* seq_start,
+                                 const void* kcache, const void* vcache, const int32_t* page_table,
+                                 int table_stride, int page_size, int ring, int n_seqs, int max_len,
+                                 int nh, int nkv, int hd, float scale, float cap, int window, void* stream);
 
 // One query row per sequence over the paged cache.  partial: float32
 // [B][nh][nsplit][hd + 2] scratch.  seq_len[b] = keys of sequence b, the new one included.
@@ -120,6 +130,12 @@ int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache, const 
                           const int32_t* page_table, int table_stride, int page_size, int ring,
                           const int32_t* seq_slot, const int32_t* seq_len, float* partial,
                           int nsplit, int waves, int B, int nh, int nkv, int hd, float scale,
+                          int window, void* stream);
+// The same with a soft cap on the scores, cap tanh(score / cap) (cap <= 0: none).
+int illm_attn_decode_bf16_cap(const void* qkv, void* out, const void* kcache, const void* vcache,
+                          const int32_t* page_table, int table_stride, int page_size, int ring,
+                          const int32_t* seq_slot, const int32_t* seq_len, float* partial,
+                          int nsplit, int waves, int B, int nh, int nkv, int hd, float scale, float cap,
                           int window, void* stream);
 
 // illm_attn_decode_bf16 for callers that cannot allocate device memory (code under HIP graph
@@ -355,8 +371,8 @@ int illm_delta_conv_tail(const void* P, int p_dt, int p_stride, void* tail, int 
                          void* stream);
 int illm_delta_scan(const float* qn, const float* kn, const float* vv, const float* beta,
                     const float* dec, int DW, float* state, const int32_t* cu,
-                    const int32_t* seq_slot, float* o, int n_seqs, int G, int H, int dk, int dv,
-                    void* stream);
+                    const int32_t* seq_slot, float* o, int n_seqs, int max_rows, int G, int H, int dk,
+                    int dv, void* stream);
 int illm_delta_finish(const float* o, const void* w, int w_dt, const void* Z, int z_dt, int z_stride,
                       int z_off, int gate_kind, void* out, int out_dt, int T, int H, int dv,
                       float eps, void* stream);

@@ -30,6 +30,14 @@ __device__ __forceinline__ float fexp(float x) {
     return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
 }
 
+// A soft cap on a score: cap * tanh(x / cap) as cap (1 - 2 / (1 + e^(2 x / cap))), by the
+// hardware's exp2 and reciprocal; cap <= 0: the score as it is.
+__device__ __forceinline__ float soft_cap_fast(float x, float cap) {
+    if (!(cap > 0.f)) return x;
+    const float e = __builtin_amdgcn_exp2f(x * (2.0f * 1.44269504088896340736f / cap));
+    return cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e));
+}
+
 __device__ __forceinline__ void unpack8(const illm_u32x4_t& v, float* f) {
     f[0] = __uint_as_float(v[0] << 16); f[1] = __uint_as_float(v[0] & 0xffff0000u);
     f[2] = __uint_as_float(v[1] << 16); f[3] = __uint_as_float(v[1] & 0xffff0000u);
@@ -110,7 +118,7 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
                         const int32_t* __restrict__ page_table, int table_stride, int page_size,
                         int ring, const int32_t* __restrict__ seq_slot,
                         const int32_t* __restrict__ seq_len, float* __restrict__ partial,
-                        int nsplit, int nh, int nkv, int hd, float scale, int window) {
+                        int nsplit, int nh, int nkv, int hd, float scale, int window, float cap) {
     constexpr int KPI = 64 / LPR;              // keys per load instruction
     constexpr int NI = LPR < 16 ? LPR : 16;    // load instructions per tile
     constexpr int TK = NI * KPI;               // keys per tile
@@ -234,7 +242,7 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
                     part[k] = keep + __shfl_xor(send, b, ILLM_WAVE);
                 }
             }
-            s_own[g] = part[0] * scale;
+            s_own[g] = soft_cap_fast(part[0] * scale, cap);
         }
         // (scheduling barriers: the compiler would move these loads down to the others)
         __builtin_amdgcn_sched_barrier(0);
@@ -351,7 +359,7 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
                             const int32_t* __restrict__ page_table, int table_stride,
                             int page_size, int ring, const int32_t* __restrict__ seq_slot,
                             const int32_t* __restrict__ seq_len, float* __restrict__ partial,
-                            int nsplit, int nh, int nkv, float scale, int window) {
+                            int nsplit, int nh, int nkv, float scale, int window, float cap) {
     constexpr int LPR = HD <= 32 ? 4 : (HD <= 64 ? 8 : (HD <= 128 ? 16 : 32));
     constexpr int KPI = 64 / LPR;
     constexpr int NI = LPR < 16 ? LPR : 16;
@@ -427,7 +435,7 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
             for (int i = 0; i < 4; ++i) {
                 const int key = k0 + sub * 16 + 4 * q4 + i;
                 const bool ok = key < len && key >= kf;
-                sv[sub][i] = ok ? a[i] * scale : NEG_INF;
+                sv[sub][i] = ok ? soft_cap_fast(a[i] * scale, cap) : NEG_INF;
                 mx = fmaxf(mx, sv[sub][i]);
             }
         }
@@ -587,7 +595,7 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
                                const int32_t* __restrict__ page_table, int table_stride,
                                int page_size, int ring, const int32_t* __restrict__ seq_slot,
                                const int32_t* __restrict__ seq_len, float* __restrict__ partial,
-                               int nsplit, int nh, int nkv, float scale, int window) {
+                               int nsplit, int nh, int nkv, float scale, int window, float cap) {
     constexpr int TK = 64;                     // keys per tile
     constexpr int KS = HD / 32;                // k-steps of 32 dims of the first product
     extern __shared__ __attribute__((aligned(16))) float lds[];   // the waves' results at the end
@@ -690,7 +698,7 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
             for (int i = 0; i < 4; ++i) {
                 const int key = k0 + sub * 16 + 4 * q4 + i;
                 const bool ok = key < len && key >= kf;
-                sv[sub][i] = ok ? a[i] * scale : NEG_INF;
+                sv[sub][i] = ok ? soft_cap_fast(a[i] * scale, cap) : NEG_INF;
                 mx = fmaxf(mx, sv[sub][i]);
             }
         }
@@ -864,7 +872,7 @@ static int launch_decode(const void* qkv, void* out, const void* kcache, const v
                          const int32_t* page_table, int table_stride, int page_size, int ring,
                          const int32_t* seq_slot, const int32_t* seq_len, float* partial,
                          int nsplit, int waves, int B, int nh, int nkv, int hd, float scale,
-                         int window, hipStream_t stream) {
+                         int window, float cap, hipStream_t stream) {
     const int G = nh / nkv;
     const int chunks = (G + GC - 1) / GC;
     const int maxw = GC <= 4 ? 8 : 4;
@@ -873,7 +881,7 @@ static int launch_decode(const void* qkv, void* out, const void* kcache, const v
     hipLaunchKernelGGL((attn_decode_bf16_kernel<LPR, GC>), dim3(nkv * chunks, B, nsplit),
                        dim3(64 * waves), smem, stream, (const bf16_t*)qkv, (bf16_t*)out, (const bf16_t*)kcache,
                        (const bf16_t*)vcache, page_table, table_stride, page_size, ring, seq_slot,
-                       seq_len, partial, nsplit, nh, nkv, hd, scale, window);
+                       seq_len, partial, nsplit, nh, nkv, hd, scale, window, cap);
     if (nsplit > 1)
         hipLaunchKernelGGL(attn_decode_bf16_merge_kernel, dim3(nh, B), dim3(64), 0, stream,
                            (const float*)partial, (bf16_t*)out, nsplit, nh, hd);
@@ -885,11 +893,12 @@ static int launch_decode_g(int gc, const void* qkv, void* out, const void* kcach
                            const void* vcache, const int32_t* page_table, int table_stride,
                            int page_size, int ring, const int32_t* seq_slot,
                            const int32_t* seq_len, float* partial, int nsplit, int waves, int B,
-                           int nh, int nkv, int hd, float scale, int window, hipStream_t stream) {
+                           int nh, int nkv, int hd, float scale, int window, float cap,
+                           hipStream_t stream) {
 #define GO(GC_)                                                                                   \
     return launch_decode<LPR, GC_>(qkv, out, kcache, vcache, page_table, table_stride, page_size, \
                                    ring, seq_slot, seq_len, partial, nsplit, waves, B, nh, nkv,  \
-                                   hd, scale, window, stream)
+                                   hd, scale, window, cap, stream)
     switch (gc) {
         case 1: GO(1);
         case 2: GO(2);
@@ -906,12 +915,13 @@ static int launch_decode_g(int gc, const void* qkv, void* out, const void* kcach
 static int GQA_PV_ON_MATRIX_CORES = 1;      // 0: the kernel with P.V on the vector units (tuning)
 extern "C" void illm_set_gqa_pv_on_matrix_cores(int on) { GQA_PV_ON_MATRIX_CORES = on; }
 
-extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache,
-                                     const void* vcache, const int32_t* page_table,
-                                     int table_stride, int page_size, int ring,
-                                     const int32_t* seq_slot, const int32_t* seq_len,
-                                     float* partial, int nsplit, int waves, int B, int nh, int nkv,
-                                     int hd, float scale, int window, void* stream) {
+extern "C" int illm_attn_decode_bf16_cap(const void* qkv, void* out, const void* kcache,
+                                         const void* vcache, const int32_t* page_table,
+                                         int table_stride, int page_size, int ring,
+                                         const int32_t* seq_slot, const int32_t* seq_len,
+                                         float* partial, int nsplit, int waves, int B, int nh,
+                                         int nkv, int hd, float scale, float cap, int window,
+                                         void* stream) {
     if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 || hd % 8 ||
         page_size <= 0 || page_size % 64 || nsplit <= 0 || nsplit > 64 || B > 65535 ||
         table_stride <= 0 || (nsplit > 1 && !partial))
@@ -928,7 +938,7 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
     hipLaunchKernelGGL((attn_decode_bf16_gqa_pv_kernel<HD_>), grid, dim3(64 * wq), smem,           \
                        (hipStream_t)stream, (const bf16_t*)qkv, (bf16_t*)out,                      \
                        (const bf16_t*)kcache, (const bf16_t*)vcache, page_table, table_stride,     \
-                       page_size, ring, seq_slot, seq_len, partial, nsplit, nh, nkv, scale, window)
+                       page_size, ring, seq_slot, seq_len, partial, nsplit, nh, nkv, scale, window, cap)
         switch (hd) {
             case 32: GQA_PV(32); break;
             case 64: GQA_PV(64); break;
@@ -962,7 +972,7 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
     hipLaunchKernelGGL((attn_decode_bf16_gqa_kernel<HD_, GC_>), grid, dim3(64 * wq), smem,         \
                        (hipStream_t)stream, (const bf16_t*)qkv, (bf16_t*)out,                      \
                        (const bf16_t*)kcache, (const bf16_t*)vcache, page_table, table_stride,     \
-                       page_size, ring, seq_slot, seq_len, partial, nsplit, nh, nkv, scale, window)
+                       page_size, ring, seq_slot, seq_len, partial, nsplit, nh, nkv, scale, window, cap)
 #define GQA_HD(HD_)                                                                                \
     do {                                                                                           \
         if (gcq == 2) GQA(HD_, 2);                                                                 \
@@ -996,7 +1006,7 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
 #define GO(LPR_)                                                                                   \
     return launch_decode_g<LPR_>(gc, qkv, out, kcache, vcache, page_table, table_stride, page_size, \
                                  ring, seq_slot, seq_len, partial, nsplit, waves, B, nh, nkv, hd,  \
-                                 scale, window, st)
+                                 scale, window, cap, st)
     switch (lpr) {
         case 1: GO(1);
         case 2: GO(2);
@@ -1013,6 +1023,17 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
 // through a file-scope array instead of a workspace argument.  Each GPU holds its own copy of the
 // array at its own address, which the host learns once per device from the runtime; host code
 // never passes the array's name to a kernel.
+extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache,
+                                     const void* vcache, const int32_t* page_table,
+                                     int table_stride, int page_size, int ring,
+                                     const int32_t* seq_slot, const int32_t* seq_len,
+                                     float* partial, int nsplit, int waves, int B, int nh, int nkv,
+                                     int hd, float scale, int window, void* stream) {
+    return illm_attn_decode_bf16_cap(qkv, out, kcache, vcache, page_table, table_stride, page_size,
+                                     ring, seq_slot, seq_len, partial, nsplit, waves, B, nh, nkv, hd,
+                                     scale, 0.f, window, stream);
+}
+
 static __device__ __align__(256) float scratch[ILLM_DECODE_SCRATCH_BYTES / sizeof(float)];
 
 #define ILLM_MAX_DEVICES 64

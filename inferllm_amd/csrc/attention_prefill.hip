@@ -50,12 +50,20 @@ struct PfPages {
     int table_stride, page_size, ring;
 };
 
+// A soft cap on a score in the exponent's units (base 2, log2(e) folded in):
+// cap tanh(x / cap) as cap (1 - 2 / (1 + e^(2 x / cap))); cap <= 0: the score as it is.
+__device__ __forceinline__ float pf_soft_cap(float x, float cap_log2) {
+    if (!(cap_log2 > 0.f)) return x;
+    const float e = __builtin_amdgcn_exp2f(x * (2.0f * 1.44269504088896340736f / cap_log2));
+    return cap_log2 * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e));
+}
+
 template <int HD, bool PAGED>
 __global__ void __launch_bounds__(256, (HD <= 128 ? 2 : 1))
 attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
                          const int32_t* __restrict__ cu, int n_qblk, int nh, int nkv,
                          float scale_log2, int window, int hb_per_xcd, int n_hb, int zigzag,
-                         PfPages pg) {
+                         PfPages pg, float cap_log2) {
     constexpr int KLD = HD + 8;        // K tile row stride: 16 bytes of padding
     constexpr int VLD = PF_BN + 4;     // V^T row stride
     constexpr int KS = HD / 16;        // k-steps of the first product
@@ -185,7 +193,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
                 for (int i = 0; i < 16; ++i) {
                     const int key = k0 + sub * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
                     const bool ok = key <= qp && key < total && (window <= 0 || key > qp - window);
-                    const float v = ok ? s[sub][i] * scale_log2 : NEG_INF;
+                    const float v = ok ? pf_soft_cap(s[sub][i] * scale_log2, cap_log2) : NEG_INF;
                     s[sub][i] = v;
                     mx = fmaxf(mx, v);
                 }
@@ -194,7 +202,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
             for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const float v = s[sub][i] * scale_log2;
+                    const float v = pf_soft_cap(s[sub][i] * scale_log2, cap_log2);
                     s[sub][i] = v;
                     mx = fmaxf(mx, v);
                 }
@@ -568,7 +576,7 @@ static int prefill2_lds_ready(size_t bytes) {
 template <int HD>
 static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_seqs, int max_len,
                           int nh, int nkv, float scale, int window, hipStream_t st,
-                          const PfPages* pg = nullptr) {
+                          const PfPages* pg = nullptr, float cap = 0.f) {
     const int n_qblk = (max_len + PF_BM - 1) / PF_BM;
     const long long n_hb = (long long)nh * n_seqs;
     const long long hb_per_xcd = (n_hb + 7) / 8;
@@ -580,7 +588,7 @@ static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_s
         // 66 -> 64; eight of 512 lose (45 -> 48: a tile more of set-up before the first product).
         // (steps that go on from the cache: `max_len` is the most rows a sequence brings, which
         // see at least as many keys)
-        if (PF_TWO_BUFFERS == 2 || (PF_TWO_BUFFERS == 1 && HD >= 64 && max_len >= 1024 && scale > 0.f)) {
+        if (PF_TWO_BUFFERS == 2 || (PF_TWO_BUFFERS == 1 && HD >= 64 && max_len >= 1024 && scale > 0.f && !(cap > 0.f))) {
             const size_t lds = (size_t)2 * (PF_BN * (HD + 8) + HD * (PF_BN + 8)) * sizeof(bf16_t);
             const int rc = pg ? prefill2_lds_ready<HD, true>(lds) : prefill2_lds_ready<HD, false>(lds);
             if (rc != ILLM_OK) return rc;
@@ -601,54 +609,55 @@ static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_s
         hipLaunchKernelGGL((attn_prefill_mfma_kernel<HD, true>), dim3((unsigned)blocks), dim3(256), 0,
                            st, (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
                            scale * 1.44269504088896340736f, window, (int)hb_per_xcd, (int)n_hb,
-                           hb_per_xcd * n_qblk <= 64 ? 1 : 0, *pg);
+                           hb_per_xcd * n_qblk <= 64 ? 1 : 0, *pg, cap * 1.44269504088896340736f);
         return illm_launch_status();
     }
     hipLaunchKernelGGL((attn_prefill_mfma_kernel<HD, false>), dim3((unsigned)blocks), dim3(256), 0, st,
                        (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
                        scale * 1.44269504088896340736f, window, (int)hb_per_xcd, (int)n_hb,
-                       hb_per_xcd * n_qblk <= 64 ? 1 : 0, PfPages());   // 32 CUs of an XCD, two blocks each
+                       hb_per_xcd * n_qblk <= 64 ? 1 : 0, PfPages(),    // 32 CUs of an XCD, two blocks each
+                       cap * 1.44269504088896340736f);
     return illm_launch_status();
 }
 
 // Takes bfloat16 and a head_dim that is a multiple of 16 up to 256; else ILLM_ERR_ARG.
-extern "C" int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t* cu_seqlens,
+extern "C" int illm_attn_prefill_bf16_cap(const void* qkv, void* out, const int32_t* cu_seqlens,
                                       int n_seqs, int max_len, int nh, int nkv, int hd,
-                                      float scale, int window, void* stream) {
+                                      float scale, float cap, int window, void* stream) {
     if (n_seqs < 0 || max_len < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 ||
         hd % 16)
         return ILLM_ERR_ARG;
     if (n_seqs == 0 || max_len == 0) return ILLM_OK;
     hipStream_t st = (hipStream_t)stream;
     switch (hd) {
-        case 32: return launch_prefill<32>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 64: return launch_prefill<64>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 96: return launch_prefill<96>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 128: return launch_prefill<128>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 160: return launch_prefill<160>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 192: return launch_prefill<192>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 224: return launch_prefill<224>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 16: return launch_prefill<16>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 48: return launch_prefill<48>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 80: return launch_prefill<80>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 112: return launch_prefill<112>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 144: return launch_prefill<144>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 176: return launch_prefill<176>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 208: return launch_prefill<208>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        case 240: return launch_prefill<240>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
-        default: return launch_prefill<256>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 32: return launch_prefill<32>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 64: return launch_prefill<64>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 96: return launch_prefill<96>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 128: return launch_prefill<128>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 160: return launch_prefill<160>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 192: return launch_prefill<192>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 224: return launch_prefill<224>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 16: return launch_prefill<16>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 48: return launch_prefill<48>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 80: return launch_prefill<80>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 112: return launch_prefill<112>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 144: return launch_prefill<144>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 176: return launch_prefill<176>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 208: return launch_prefill<208>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        case 240: return launch_prefill<240>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
+        default: return launch_prefill<256>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, nullptr, cap);
     }
 }
 
 // The same where the step's rows go on from tokens the cache already holds: keys and values from
 // the paged cache (bfloat16, pages of a multiple of 64 rows), row r of sequence b at position
 // seq_start[b] + r.  The step's own keys and values must be in the cache already.
-extern "C" int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const int32_t* cu_seqlens,
+extern "C" int illm_attn_prefill_paged_bf16_cap(const void* qkv, void* out, const int32_t* cu_seqlens,
                                             const int32_t* seq_slot, const int32_t* seq_start,
                                             const void* kcache, const void* vcache,
                                             const int32_t* page_table, int table_stride,
                                             int page_size, int ring, int n_seqs, int max_len, int nh,
-                                            int nkv, int hd, float scale, int window, void* stream) {
+                                            int nkv, int hd, float scale, float cap, int window, void* stream) {
     if (n_seqs < 0 || max_len < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 ||
         hd % 16 || !seq_slot || !seq_start || !kcache || !vcache || !page_table ||
         table_stride <= 0 || page_size <= 0 || page_size % PF_BN)
@@ -658,21 +667,37 @@ extern "C" int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const in
     const PfPages pg = {(const bf16_t*)kcache, (const bf16_t*)vcache, page_table, seq_slot, seq_start,
                         table_stride, page_size, ring};
     switch (hd) {
-        case 32: return launch_prefill<32>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 64: return launch_prefill<64>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 96: return launch_prefill<96>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 128: return launch_prefill<128>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 160: return launch_prefill<160>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 192: return launch_prefill<192>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 224: return launch_prefill<224>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 16: return launch_prefill<16>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 48: return launch_prefill<48>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 80: return launch_prefill<80>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 112: return launch_prefill<112>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 144: return launch_prefill<144>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 176: return launch_prefill<176>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 208: return launch_prefill<208>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        case 240: return launch_prefill<240>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
-        default: return launch_prefill<256>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 32: return launch_prefill<32>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 64: return launch_prefill<64>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 96: return launch_prefill<96>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 128: return launch_prefill<128>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 160: return launch_prefill<160>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 192: return launch_prefill<192>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 224: return launch_prefill<224>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 16: return launch_prefill<16>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 48: return launch_prefill<48>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 80: return launch_prefill<80>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 112: return launch_prefill<112>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 144: return launch_prefill<144>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 176: return launch_prefill<176>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 208: return launch_prefill<208>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        case 240: return launch_prefill<240>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
+        default: return launch_prefill<256>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg, cap);
     }
+}
+
+// The same without a cap on the scores.
+extern "C" int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t* cu_seqlens,
+                                      int n_seqs, int max_len, int nh, int nkv, int hd,
+                                      float scale, int window, void* stream) {
+    return illm_attn_prefill_bf16_cap(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, hd, scale, 0.f, window, stream);
+}
+
+extern "C" int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const int32_t* cu_seqlens,
+                                            const int32_t* seq_slot, const int32_t* seq_start,
+                                            const void* kcache, const void* vcache,
+                                            const int32_t* page_table, int table_stride,
+                                            int page_size, int ring, int n_seqs, int max_len, int nh,
+                                            int nkv, int hd, float scale, int window, void* stream) {
+    return illm_attn_prefill_paged_bf16_cap(qkv, out, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table, table_stride, page_size, ring, n_seqs, max_len, nh, nkv, hd, scale, 0.f, window, stream);
 }

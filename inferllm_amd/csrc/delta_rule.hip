@@ -132,19 +132,41 @@ extern "C" int illm_delta_conv_tail(const void* P, int p_dt, int p_stride, void*
     return illm_launch_status();
 }
 
-// The recurrence.  grid (ceil(dv / 16), H, sequences); one wave: lane = column + 16 part; a lane
-// holds rows [part NS, part NS + NS) of its column of S, so S^T k and S^T q are NS multiply-adds
-// and two exchanges a lane.  The next token's k, q and decays are asked for before this token's
-// arithmetic.  state [slots][H][dk][dv] float32.
-template <int NS>
+// The recurrence.  grid (ceil(dv / COLS), H, sequences), COLS = 64 / PARTS; one wave: lane = part +
+// PARTS * column; a lane holds rows [part NS, part NS + NS) of its column of S, so S^T k and S^T q
+// are NS multiply-adds a lane and a sum over the PARTS neighbouring lanes, which stays inside a
+// row of 16 lanes (data-parallel moves, no trip through LDS).  Long sequences take 16 parts (the
+// chain of dependent operations a token is what bounds them), steps of few tokens take 4 (the
+// state's rows are then read and written 64 bytes a piece).  The next token's k, q and decays are
+// asked for before this token's arithmetic.  state [slots][H][dk][dv] float32.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+
+// The sum over the PARTS lanes of a group; every lane of the group gets the same bits.
+template <int PARTS>
+__device__ __forceinline__ float group_sum(float v) {
+    v += dpp_move<0xB1>(v);                 // lanes 1 0 3 2 of every four
+    v += dpp_move<0x4E>(v);                 // lanes 2 3 0 1
+    if (PARTS == 16) {
+        v += dpp_move<0x141>(v);            // the other four of every eight (mirrored)
+        v += dpp_move<0x140>(v);            // the other eight of the sixteen (mirrored)
+    }
+    return v;
+}
+
+template <int NS, int PARTS>
 __global__ void __launch_bounds__(64)
 delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                   const float* __restrict__ vv, const float* __restrict__ beta,
                   const float* __restrict__ dec, int DW, float* __restrict__ state,
                   const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_slot,
                   float* __restrict__ o, int G, int H, int dk, int dv) {
+    constexpr int COLS = 64 / PARTS;
+    constexpr int NA = NS >= 4 ? 4 : NS;                // partial sums, to keep the chains short
     const int b = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
-    const int col = blockIdx.x * 16 + (lane & 15), part = lane >> 4;
+    const int part = lane % PARTS, col = blockIdx.x * COLS + lane / PARTS;
     const int r0 = cu[b], n = cu[b + 1] - r0;
     if (n <= 0) return;
     const int slot = seq_slot[b], gh = h / (H / G), i0 = part * NS;
@@ -153,75 +175,212 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
     float s[NS], kc[NS], qc[NS], gc[NS];
 #pragma unroll
     for (int ii = 0; ii < NS; ++ii) s[ii] = (live && i0 + ii < dk) ? sp[(size_t)(i0 + ii) * dv] : 0.f;
-    auto fetch = [&](int row, float* k_, float* q_, float* g_, float& v_, float& b_) {
-        const float* kp = kn + ((size_t)row * G + gh) * dk;
-        const float* qp = qn + ((size_t)row * G + gh) * dk;
-        const float* dp = dec + ((size_t)row * H + h) * DW;
-#pragma unroll
-        for (int ii = 0; ii < NS; ++ii) {
-            const int i = i0 + ii;
-            const bool in = i < dk;
-            k_[ii] = in ? kp[i] : 0.f;
-            q_[ii] = in ? qp[i] : 0.f;
-            g_[ii] = in ? (DW == 1 ? dp[0] : dp[i]) : 1.f;
-        }
-        v_ = live ? vv[((size_t)row * H + h) * dv + col] : 0.f;
-        b_ = beta[(size_t)row * H + h];
-    };
     float vc, bc;
-    fetch(r0, kc, qc, gc, vc, bc);
+#define DELTA_FETCH(ROW, K_, Q_, G_, V_, B_)                                                      \
+    {                                                                                             \
+        const float* kp = kn + ((size_t)(ROW) * G + gh) * dk;                                     \
+        const float* qp = qn + ((size_t)(ROW) * G + gh) * dk;                                     \
+        const float* dp = dec + ((size_t)(ROW) * H + h) * DW;                                     \
+        _Pragma("unroll") for (int ii = 0; ii < NS; ++ii) {                                       \
+            const int i = i0 + ii;                                                                \
+            const bool in = i < dk;                                                               \
+            K_[ii] = in ? kp[i] : 0.f;                                                            \
+            Q_[ii] = in ? qp[i] : 0.f;                                                            \
+            G_[ii] = in ? (DW == 1 ? dp[0] : dp[i]) : 1.f;                                        \
+        }                                                                                         \
+        V_ = live ? vv[((size_t)(ROW) * H + h) * dv + col] : 0.f;                                 \
+        B_ = beta[(size_t)(ROW) * H + h];                                                         \
+    }
+    DELTA_FETCH(r0, kc, qc, gc, vc, bc)
     for (int t = 0; t < n; ++t) {
         const int row = r0 + t;
         float kx[NS], qx[NS], gx[NS], vx, bx;
-        fetch(t + 1 < n ? row + 1 : row, kx, qx, gx, vx, bx);
-        float kv = 0.f;
+        const int nxt = t + 1 < n ? row + 1 : row;
+        DELTA_FETCH(nxt, kx, qx, gx, vx, bx)
+        float pa[NA];
+#pragma unroll
+        for (int a = 0; a < NA; ++a) pa[a] = 0.f;
 #pragma unroll
         for (int ii = 0; ii < NS; ++ii) {
             s[ii] *= gc[ii];
-            kv = fmaf(s[ii], kc[ii], kv);
+            pa[ii % NA] = fmaf(s[ii], kc[ii], pa[ii % NA]);
         }
-        kv += __shfl_xor(kv, 16, 64);
-        kv += __shfl_xor(kv, 32, 64);
+        float kv = pa[0];
+#pragma unroll
+        for (int a = 1; a < NA; ++a) kv += pa[a];
+        kv = group_sum<PARTS>(kv);
         const float u = bc * (vc - kv);
-        float ov = 0.f;
+#pragma unroll
+        for (int a = 0; a < NA; ++a) pa[a] = 0.f;
 #pragma unroll
         for (int ii = 0; ii < NS; ++ii) {
             s[ii] = fmaf(kc[ii], u, s[ii]);
-            ov = fmaf(s[ii], qc[ii], ov);
+            pa[ii % NA] = fmaf(s[ii], qc[ii], pa[ii % NA]);
         }
-        ov += __shfl_xor(ov, 16, 64);
-        ov += __shfl_xor(ov, 32, 64);
+        float ov = pa[0];
+#pragma unroll
+        for (int a = 1; a < NA; ++a) ov += pa[a];
+        ov = group_sum<PARTS>(ov);
         if (part == 0 && live) o[((size_t)row * H + h) * dv + col] = ov;
 #pragma unroll
         for (int ii = 0; ii < NS; ++ii) { kc[ii] = kx[ii]; qc[ii] = qx[ii]; gc[ii] = gx[ii]; }
         vc = vx; bc = bx;
     }
+#undef DELTA_FETCH
 #pragma unroll
     for (int ii = 0; ii < NS; ++ii)
         if (live && i0 + ii < dk) sp[(size_t)(i0 + ii) * dv] = s[ii];
 }
 
+// The same recurrence for long runs of tokens (16 parts a column, part p holding rows p, p + 16, ...).  What bounds it is the chain of
+// dependent operations a token, so nothing may wait for memory inside it: the k, q and decay rows of
+// DELTA_CHUNK tokens go through LDS in two buffers, the next chunk's loads (and its v and beta, in
+// registers) are issued before this chunk's arithmetic and stored after it.  One wave a block;
+// dynamic LDS: 2 * DELTA_CHUNK * (2 dk + DW) floats.
+#define DELTA_CHUNK 8
+template <int NS>
+__global__ void __launch_bounds__(64)
+delta_scan_long_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
+                       const float* __restrict__ vv, const float* __restrict__ beta,
+                       const float* __restrict__ dec, int DW, float* __restrict__ state,
+                       const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_slot,
+                       float* __restrict__ o, int G, int H, int dk, int dv) {
+    constexpr int PARTS = 16, COLS = 4, TC = DELTA_CHUNK;
+    constexpr int JJ = NS >= 4 ? NS / 4 : 1;            // pieces of 64 floats in a row of 16 NS
+    constexpr int NA = NS >= 4 ? 4 : NS;
+    extern __shared__ float stage[];
+    const int b = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
+    const int part = lane % PARTS, col = blockIdx.x * COLS + lane / PARTS;
+    const int r0 = cu[b], n = cu[b + 1] - r0;
+    if (n <= 0) return;
+    const int slot = seq_slot[b], gh = h / (H / G);
+    const bool live = col < dv;
+    const int RW = 2 * dk + DW;
+    float* sp = state + (((size_t)slot * H + h) * dk) * dv + col;
+    float s[NS];
+#pragma unroll
+    for (int ii = 0; ii < NS; ++ii)      // row part + 16 ii: the 16 parts read neighbouring words of LDS
+        s[ii] = (live && part + PARTS * ii < dk) ? sp[(size_t)(part + PARTS * ii) * dv] : 0.f;
+    float sk[TC][JJ], sq[TC][JJ], sg[TC][JJ], sv[TC], sb[TC];
+#define DELTA_LOAD(T0)                                                                            \
+    _Pragma("unroll") for (int tt = 0; tt < TC; ++tt) {                                           \
+        const int row = r0 + ((T0) + tt < n ? (T0) + tt : n - 1);                                 \
+        const float* kp = kn + ((size_t)row * G + gh) * dk;                                       \
+        const float* qp = qn + ((size_t)row * G + gh) * dk;                                       \
+        const float* dp = dec + ((size_t)row * H + h) * DW;                                       \
+        _Pragma("unroll") for (int jj = 0; jj < JJ; ++jj) {                                       \
+            const int j = lane + 64 * jj;                                                         \
+            sk[tt][jj] = j < dk ? kp[j] : 0.f;                                                    \
+            sq[tt][jj] = j < dk ? qp[j] : 0.f;                                                    \
+            sg[tt][jj] = j < DW ? dp[j] : 1.f;                                                    \
+        }                                                                                         \
+        sv[tt] = live ? vv[((size_t)row * H + h) * dv + col] : 0.f;                               \
+        sb[tt] = beta[(size_t)row * H + h];                                                       \
+    }
+#define DELTA_STORE(BUF)                                                                          \
+    _Pragma("unroll") for (int tt = 0; tt < TC; ++tt) {                                           \
+        float* dst = stage + ((size_t)(BUF) * TC + tt) * RW;                                      \
+        _Pragma("unroll") for (int jj = 0; jj < JJ; ++jj) {                                       \
+            const int j = lane + 64 * jj;                                                         \
+            if (j < dk) { dst[j] = sk[tt][jj]; dst[dk + j] = sq[tt][jj]; }                        \
+            if (j < DW) dst[2 * dk + j] = sg[tt][jj];                                             \
+        }                                                                                         \
+    }
+    DELTA_LOAD(0)
+    DELTA_STORE(0)
+    __syncthreads();
+    for (int t0 = 0, buf = 0; t0 < n; t0 += TC, buf ^= 1) {
+        float cv[TC], cb[TC];
+#pragma unroll
+        for (int tt = 0; tt < TC; ++tt) { cv[tt] = sv[tt]; cb[tt] = sb[tt]; }
+        const bool more = t0 + TC < n;
+        if (more) DELTA_LOAD(t0 + TC)
+#pragma unroll
+        for (int tt = 0; tt < TC; ++tt) {
+            if (t0 + tt < n) {
+                const float* src = stage + ((size_t)buf * TC + tt) * RW;
+                float kc[NS], qc[NS], gc[NS];
+#pragma unroll
+                for (int ii = 0; ii < NS; ++ii) {
+                    const int i = part + PARTS * ii;
+                    const bool in = i < dk;
+                    kc[ii] = in ? src[i] : 0.f;
+                    qc[ii] = in ? src[dk + i] : 0.f;
+                    gc[ii] = in ? src[2 * dk + (DW == 1 ? 0 : i)] : 1.f;
+                }
+                float pa[NA];
+#pragma unroll
+                for (int a = 0; a < NA; ++a) pa[a] = 0.f;
+#pragma unroll
+                for (int ii = 0; ii < NS; ++ii) {
+                    s[ii] *= gc[ii];
+                    pa[ii % NA] = fmaf(s[ii], kc[ii], pa[ii % NA]);
+                }
+                float kv = pa[0];
+#pragma unroll
+                for (int a = 1; a < NA; ++a) kv += pa[a];
+                kv = group_sum<PARTS>(kv);
+                const float u = cb[tt] * (cv[tt] - kv);
+#pragma unroll
+                for (int a = 0; a < NA; ++a) pa[a] = 0.f;
+#pragma unroll
+                for (int ii = 0; ii < NS; ++ii) {
+                    s[ii] = fmaf(kc[ii], u, s[ii]);
+                    pa[ii % NA] = fmaf(s[ii], qc[ii], pa[ii % NA]);
+                }
+                float ov = pa[0];
+#pragma unroll
+                for (int a = 1; a < NA; ++a) ov += pa[a];
+                ov = group_sum<PARTS>(ov);
+                if (part == 0 && live) o[((size_t)(r0 + t0 + tt) * H + h) * dv + col] = ov;
+            }
+        }
+        if (more) DELTA_STORE(buf ^ 1)
+        __syncthreads();
+    }
+#undef DELTA_LOAD
+#undef DELTA_STORE
+#pragma unroll
+    for (int ii = 0; ii < NS; ++ii)
+        if (live && part + PARTS * ii < dk) sp[(size_t)(part + PARTS * ii) * dv] = s[ii];
+}
+
+// `max_rows`: the most rows a sequence of the step has.  It chooses the layout (16 parts from 16
+// rows on), and the layout the order of a row's sums: a row of a long step and the same row as a
+// single token differ in rounding, in nothing else.
 extern "C" int illm_delta_scan(const float* qn, const float* kn, const float* vv, const float* beta,
                                const float* dec, int DW, float* state, const int32_t* cu,
-                               const int32_t* seq_slot, float* o, int n_seqs, int G, int H, int dk,
-                               int dv, void* stream) {
+                               const int32_t* seq_slot, float* o, int n_seqs, int max_rows, int G,
+                               int H, int dk, int dv, void* stream) {
     if (n_seqs < 0 || G <= 0 || H <= 0 || H % G || dk <= 0 || dk > 256 || dv <= 0 ||
         (DW != 1 && DW != dk) || H > 65535 || n_seqs > 65535)
         return ILLM_ERR_ARG;
     if (n_seqs == 0) return ILLM_OK;
-    const dim3 grid((dv + 15) / 16, H, n_seqs);
     hipStream_t st = (hipStream_t)stream;
-#define GO(NS_)                                                                                  \
-    hipLaunchKernelGGL(delta_scan_kernel<NS_>, grid, dim3(64), 0, st, qn, kn, vv, beta, dec, DW, \
+#define GO(NS_, PARTS_)                                                                          \
+    hipLaunchKernelGGL((delta_scan_kernel<NS_, PARTS_>), dim3((dv + 64 / PARTS_ - 1) / (64 / PARTS_), H, n_seqs), \
+                       dim3(64), 0, st, qn, kn, vv, beta, dec, DW, state, cu, seq_slot, o, G, H, dk, dv)
+    if (max_rows >= 16) {
+        const int ns = (dk + 15) / 16;
+        const size_t lds = (size_t)2 * DELTA_CHUNK * (2 * dk + DW) * sizeof(float);
+        const dim3 grid((dv + 3) / 4, H, n_seqs);
+#define GOL(NS_)                                                                                  \
+    hipLaunchKernelGGL(delta_scan_long_kernel<NS_>, grid, dim3(64), lds, st, qn, kn, vv, beta, dec, DW, \
                        state, cu, seq_slot, o, G, H, dk, dv)
-    const int ns = (dk + 3) / 4;
-    if (ns <= 4) GO(4);
-    else if (ns <= 8) GO(8);
-    else if (ns <= 16) GO(16);
-    else if (ns <= 24) GO(24);
-    else if (ns <= 32) GO(32);
-    else if (ns <= 48) GO(48);
-    else GO(64);
+        if (ns <= 1) GOL(1);
+        else if (ns <= 2) GOL(2);
+        else if (ns <= 4) GOL(4);
+        else if (ns <= 8) GOL(8);
+        else GOL(16);
+#undef GOL
+    } else {
+        const int ns = (dk + 3) / 4;
+        if (ns <= 4) GO(4, 4);
+        else if (ns <= 8) GO(8, 4);
+        else if (ns <= 16) GO(16, 4);
+        else if (ns <= 32) GO(32, 4);
+        else GO(64, 4);
+    }
 #undef GO
     return illm_launch_status();
 }

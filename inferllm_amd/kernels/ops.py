@@ -1002,8 +1002,9 @@ def gate_up_silu(x, w_gate_up) -> torch.Tensor:
 
 # ------------------------------------------------------------------ attention
 def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_len: int, nh: int,
-                 nkv: int, hd: int, scale: float, window: int) -> torch.Tensor:
-    """Causal attention of whole prompts over packed rows; returns [T, nh * hd]."""
+                 nkv: int, hd: int, scale: float, window: int, softcap: float = 0.0) -> torch.Tensor:
+    """Causal attention of whole prompts over packed rows; returns [T, nh * hd].  `softcap` > 0:
+    scores softcap * tanh(score / softcap) (the matrix-core kernels only)."""
     _gpu(qkv, cu_seqlens)
     _i32(cu_seqlens, n_seqs + 1)
     T = qkv.shape[0]
@@ -1011,10 +1012,12 @@ def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_l
     _need(nh % nkv == 0, "attn_prefill: heads must be a multiple of kv heads")
     out = torch.empty((T, nh * hd), dtype=qkv.dtype, device=qkv.device)
     if qkv.dtype == torch.bfloat16 and hd % 16 == 0:
-        _check(_lib().illm_attn_prefill_bf16(
+        _check(_lib().illm_attn_prefill_bf16_cap(
             _p(qkv), _p(out), _p(cu_seqlens), n_seqs, max_len, nh, nkv, hd,
-            ctypes.c_float(scale), window, _stream()), f"attn_prefill_bf16 (head_dim {hd})")
+            ctypes.c_float(scale), ctypes.c_float(softcap), window, _stream()),
+            f"attn_prefill_bf16 (head_dim {hd})")
         return out
+    _need(not softcap, "attn_prefill: a soft cap needs bfloat16 and a head size in steps of 16")
     _check(_lib().illm_attn_prefill_generic(
         _p(qkv), _p(out), _code(qkv), _p(cu_seqlens), n_seqs, max_len, nh, nkv, hd,
         ctypes.c_float(scale), window, _stream()), f"attn_prefill (head_dim {hd})")
@@ -1025,7 +1028,7 @@ def attn_prefill_paged(qkv: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: to
                        seq_start: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                        page_table: torch.Tensor, page_size: int, ring: int, n_seqs: int,
                        max_len: int, nh: int, nkv: int, hd: int, scale: float,
-                       window: int) -> torch.Tensor:
+                       window: int, softcap: float = 0.0) -> torch.Tensor:
     """Causal attention of a step's packed rows that go on from tokens the cache already holds:
     row r of sequence b stands at position seq_start[b] + r and attends over the keys 0 .. its
     position of the paged cache, which must hold the step's own keys and values too by now.
@@ -1041,11 +1044,13 @@ def attn_prefill_paged(qkv: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: to
     _need(qkv.shape[1] == (nh + 2 * nkv) * hd, "attn_prefill_paged: packed qkv rows")
     out = torch.empty((T, nh * hd), dtype=qkv.dtype, device=qkv.device)
     if qkv.dtype == torch.bfloat16 and hd % 16 == 0 and page_size % 64 == 0:
-        _check(_lib().illm_attn_prefill_paged_bf16(
+        _check(_lib().illm_attn_prefill_paged_bf16_cap(
             _p(qkv), _p(out), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache), _p(vcache),
             _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_len, nh, nkv, hd,
-            ctypes.c_float(scale), window, _stream()), f"attn_prefill_paged_bf16 (head_dim {hd})")
+            ctypes.c_float(scale), ctypes.c_float(softcap), window, _stream()),
+            f"attn_prefill_paged_bf16 (head_dim {hd})")
         return out
+    _need(not softcap, "attn_prefill_paged: a soft cap needs bfloat16 and a head size in steps of 16")
     _check(_lib().illm_attn_prefill_paged_generic(
         _p(qkv), _p(out), _code(qkv), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
         _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_len, nh, nkv,
@@ -1080,7 +1085,7 @@ def decode_splits(B: int, nkv: int, max_len: int, nh: int = 0, hd: int = 0, ragg
 def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                 page_table: torch.Tensor, page_size: int, ring: int, seq_slot: torch.Tensor,
                 seq_len: torch.Tensor, nh: int, nkv: int, hd: int, scale: float, window: int,
-                nsplit: int, waves: int = 1) -> torch.Tensor:
+                nsplit: int, waves: int = 1, softcap: float = 0.0) -> torch.Tensor:
     """One new token per sequence against the paged cache; returns [B, nh * hd].
     seq_len[b]: keys of sequence b, the new one included.  The keys of a sequence are cut
     into `nsplit` ranges (blocks, combined by a merge kernel) and each range is shared by
@@ -1096,11 +1101,13 @@ def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
     if qkv.dtype == torch.bfloat16 and hd % 8 == 0 and page_size % 64 == 0:
         partial = (torch.empty((B, nh, nsplit, hd + 2), dtype=torch.float32, device=qkv.device)
                    if nsplit > 1 else None)
-        _check(_lib().illm_attn_decode_bf16(
+        _check(_lib().illm_attn_decode_bf16_cap(
             _p(qkv), _p(out), _p(kcache), _p(vcache), _p(page_table), page_table.shape[1],
             page_size, ring, _p(seq_slot), _p(seq_len), _p(partial), nsplit, waves, B, nh, nkv, hd,
-            ctypes.c_float(scale), window, _stream()), f"attn_decode_bf16 (head_dim {hd})")
+            ctypes.c_float(scale), ctypes.c_float(softcap), window, _stream()),
+            f"attn_decode_bf16 (head_dim {hd})")
         return out
+    _need(not softcap, "attn_decode: a soft cap needs bfloat16 and a head size in steps of 8")
     partial = torch.empty((B, nh, nsplit, hd + 2), dtype=torch.float32, device=qkv.device)
     _check(_lib().illm_attn_decode_generic(
         _p(qkv), _p(out), _code(qkv), _p(kcache), _p(vcache), _p(page_table), page_table.shape[1],
@@ -1456,26 +1463,12 @@ def attn_cap_rows(q: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Ten
     _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs); _i32(seq_start, n_seqs); _i32(page_table)
     _cap_cache_ok(q, kcache, vcache, page_table, page_size, nh, nkv, dk, dv, "attn_cap_rows")
     out = torch.empty((q.shape[0], nh * dv), dtype=q.dtype, device=q.device)
-    if (q.dtype == torch.bfloat16 and attn_cap_mfma_fits(dk, dv, page_size)):
-        _check(_lib().illm_attn_cap_rows_bf16(
-            _p(q), q.shape[1], _p(out), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
-            _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_rows, nh,
-            nkv, dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _stream()),
-            f"attn_cap_rows_bf16 (sizes {dk}, {dv})")
-        return out
     _check(_lib().illm_attn_cap_rows(
         _p(q), q.shape[1], _p(out), _code(q), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
         _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_rows, nh, nkv,
         dk, dv, ctypes.c_float(scale), ctypes.c_float(cap), window, _stream()),
         f"attn_cap_rows (sizes {dk}, {dv})")
     return out
-
-
-ATTN_CAP_MFMA = False
-
-
-def attn_cap_mfma_fits(dk: int, dv: int, page_size: int) -> bool:
-    return ATTN_CAP_MFMA and dk % 16 == 0 and dv % 16 == 0 and page_size % 64 == 0
 
 
 def attn_cap_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
@@ -1548,10 +1541,11 @@ def delta_conv_tail(P: torch.Tensor, tail: torch.Tensor, cu_seqlens: torch.Tenso
 
 
 def delta_scan(qn, kn, vv, beta, dec, state: torch.Tensor, cu_seqlens: torch.Tensor,
-               seq_slot: torch.Tensor, n_seqs: int) -> torch.Tensor:
+               seq_slot: torch.Tensor, n_seqs: int, max_rows: int) -> torch.Tensor:
     """The recurrence S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q over every
     sequence's rows in order, from `state` float32 [slots, H, dk, dv] and back into it.
-    Returns o float32 [T, H, dv]."""
+    `max_rows`: the most rows a sequence brings (long sequences are laid out for their chain of
+    tokens, short steps for the state's bytes).  Returns o float32 [T, H, dv]."""
     _gpu(qn, kn, vv, beta, dec, state, cu_seqlens, seq_slot)
     _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs)
     T, G, dk = qn.shape
@@ -1561,7 +1555,8 @@ def delta_scan(qn, kn, vv, beta, dec, state: torch.Tensor, cu_seqlens: torch.Ten
           and dec.shape[2] in (1, dk) and state.shape[1:] == (H, dk, dv), "delta_scan: shapes")
     o = torch.empty((T, H, dv), dtype=torch.float32, device=qn.device)
     _check(_lib().illm_delta_scan(_p(qn), _p(kn), _p(vv), _p(beta), _p(dec), dec.shape[2], _p(state),
-                                  _p(cu_seqlens), _p(seq_slot), _p(o), n_seqs, G, H, dk, dv, _stream()),
+                                  _p(cu_seqlens), _p(seq_slot), _p(o), n_seqs, max_rows, G, H, dk, dv,
+                                  _stream()),
            "delta_scan")
     return o
 

@@ -191,10 +191,27 @@ class CappedAttention(Mixer):
         if writes_cache:
             ops.kv_store2(qkv, nh * dk, (nh + nkv) * dk, ctx.row_pos, ctx.row_slot, kc, vc, group.table,
                           group.page_size, group.ring, nkv, dk, dv)
-        if ctx.prefill:
+        # keys and values of one width in bfloat16: the library's matrix-core attention, which
+        # takes the cap; any other sizes, and float32: the kernels of this attention's own
+        shared = qkv.dtype == torch.bfloat16 and dk == dv and dk % 16 == 0 and group.page_size % 64 == 0
+        if ctx.prefill and shared and not ctx.continues:
+            o = ops.attn_prefill(qkv, ctx.cu_seqlens, ctx.n_seqs, ctx.max_len, nh, nkv, dk, self.scale,
+                                 window, self.softcap)
+        elif ctx.prefill and shared:
+            o = ops.attn_prefill_paged(qkv, ctx.cu_seqlens, ctx.seq_slot, ctx.seq_start, kc, vc,
+                                       group.table, group.page_size, group.ring, ctx.n_seqs,
+                                       ctx.max_rows, nh, nkv, dk, self.scale, window, self.softcap)
+        elif ctx.prefill:
             o = ops.attn_cap_rows(qkv, ctx.cu_seqlens, ctx.seq_slot, ctx.seq_start, kc, vc, group.table,
                                   group.page_size, group.ring, ctx.n_seqs, ctx.max_rows, nh, nkv, dk,
                                   dv, self.scale, self.softcap, window)
+        elif shared:
+            longest = min(ctx.max_len, window) if window else ctx.max_len
+            nsplit, waves = ops.decode_splits(ctx.n_seqs, nkv, longest, nh, dk,
+                                              ragged=ctx.ragged and not window)
+            o = ops.attn_decode(qkv, kc, vc, group.table, group.page_size, group.ring, ctx.seq_slot,
+                                ctx.seq_len, nh, nkv, dk, self.scale, window, nsplit, waves,
+                                self.softcap)
         else:
             longest = min(ctx.max_len, window) if window else ctx.max_len
             tiles = max(1, (longest + 63) // 64)

@@ -123,7 +123,8 @@ class GatedDeltaRule(Mixer):
             P, self.b_off, P2 if self.ra else P, self.a_off, self.conv_w, tail, ctx.row_slot,
             self.a_log, self.dt_bias, self.G, self.H, self.dk, self.dv, self.per_channel)
         ops.delta_conv_tail(P, tail, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs, self.taps)
-        o = ops.delta_scan(qn, kn, vv, beta, dec, S, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs)
+        o = ops.delta_scan(qn, kn, vv, beta, dec, S, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs,
+                           ctx.max_rows if ctx.prefill else 1)
         y = ops.delta_finish(o, self.norm_w, P2 if self.rg else P, self.z_off, self.gate, self.eps,
                              ctx.act_dtype)
         return ops.linear(y, self.w_o)

@@ -32,7 +32,9 @@ class TokenEmbedding(Embedding):
         self.weight = self._take(tensors, "weight").contiguous()
 
     def forward(self, ctx: StepContext):
-        return ops.embed(ctx.tokens, self.weight, self.scale, self.streams)
+        if self.streams:
+            return ops.embed(ctx.tokens, self.weight, self.scale, self.streams)
+        return ops.embed(ctx.tokens, self.weight, self.scale)
 
 
 @register_part("head", "lm_head")

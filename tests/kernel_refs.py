@@ -15,7 +15,12 @@ import torch
 F64 = torch.float64
 
 
-def embed(tokens, table, scale=1.0):
+def embed(tokens, table, scale=1.0, copies=0):
+    rows = _embed_rows(tokens, table, scale)
+    return rows[:, None, :].repeat(1, copies, 1).contiguous() if copies else rows
+
+
+def _embed_rows(tokens, table, scale=1.0):
     return table[tokens.long()].to(torch.float32) * scale
 
 
@@ -116,7 +121,8 @@ def _attend(q, k, v, scale, visible):
     return out
 
 
-def attn_prefill(qkv, cu_seqlens, n_seqs, max_len, nh, nkv, hd, scale, window):
+def attn_prefill(qkv, cu_seqlens, n_seqs, max_len, nh, nkv, hd, scale, window, softcap=0.0):
+    assert not softcap
     T = qkv.shape[0]
     view = qkv.view(T, nh + 2 * nkv, hd)
     out = torch.zeros(T, nh * hd, dtype=qkv.dtype, device=qkv.device)
@@ -362,19 +368,19 @@ def few_outputs_f32(x, w):
     return (x.to(F64) @ w.to(F64).t()).to(torch.float32)
 
 
-def moe_route(z, correction, top):
-    s = torch.softmax(z.to(F64), dim=-1)
+def moe_route(z, correction, top, score="softmax"):
+    s = torch.softmax(z.to(F64), dim=-1) if score == "softmax" else torch.sigmoid(z.to(F64))
     pick = s + correction.to(F64) if correction is not None else s
     idx = torch.topk(pick, top, dim=-1).indices
     return idx.to(torch.int32), torch.gather(s, 1, idx).to(torch.float32)
 
 
-def moe_plan(h, w_router, correction, top, w_gate_up):
-    idx, wt = moe_route(few_outputs_f32(h, w_router), correction, top)
+def moe_plan(h, w_router, correction, top, w_gate_up, score="softmax"):
+    idx, wt = moe_route(few_outputs_f32(h, w_router), correction, top, score)
     return idx, wt, None
 
 
-def moe_experts(h, idx, w_gate_up, w_down, grouped=None):
+def moe_experts(h, idx, w_gate_up, w_down, grouped=None, activation="silu", limit=0.0, input_weight=None):
     T, top = idx.shape
     F = w_gate_up.shape[1] // 2
     y = torch.zeros((T * top, h.shape[1]), dtype=h.dtype)
@@ -382,8 +388,14 @@ def moe_experts(h, idx, w_gate_up, w_down, grouped=None):
         for k in range(top):
             e = int(idx[t, k])
             if e < w_gate_up.shape[0]:
-                gu = w_gate_up[e].to(F64) @ h[t].to(F64)
-                y[t * top + k] = (w_down[e].to(F64) @ (torch.nn.functional.silu(gu[:F]) * gu[F:])).to(h.dtype)
+                x = h[t].to(F64) * (input_weight[t, k].to(F64) if input_weight is not None else 1.0)
+                gu = w_gate_up[e].to(F64) @ x
+                if activation == "silu":
+                    a = torch.nn.functional.silu(gu[:F]) * gu[F:]
+                else:
+                    g, u = torch.clamp(gu[:F], max=limit), torch.clamp(gu[F:], -limit, limit)
+                    a = g * torch.sigmoid(1.702 * g) * (u + 1)
+                y[t * top + k] = (w_down[e].to(F64) @ a).to(h.dtype)
     return y
 
 
@@ -393,11 +405,142 @@ def moe_combine(h, idx, wt, y, n_real, shared=None, shared_gate=None):
     for t in range(T):
         for k in range(top):
             v = y[t * top + k] if int(idx[t, k]) < n_real else h[t]
-            out[t] += wt[t, k].to(F64) * v.to(F64)
+            out[t] += (wt[t, k].to(F64) if wt is not None else 1.0) * v.to(F64)
     if shared is not None:
         g = torch.sigmoid(h.to(F64) @ shared_gate.to(F64))[:, None] if shared_gate is not None else 1.0
         out = out + g * shared.to(F64)
     return out.to(torch.float32)
+
+
+# ---------------------------------------------------------------- several residual streams
+def stream_mix_norm(x, write, read, weight, eps, out_dtype, row_idx=None):
+    T, S, E = x.shape
+    xn = x.to(F64)
+    if write is not None:
+        y = write.ya * write.y.to(F64) + (write.yb * write.y2.to(F64) if write.y2 is not None else 0.0)
+        xn = torch.stack([sum(write.mix[s, t].to(F64) * xn[:, s] for s in range(S)) + write.out[t].to(F64) * y
+                          for t in range(S)], dim=1)
+        if row_idx is None:
+            x.copy_(xn.to(torch.float32))
+    u = sum((read[s].to(F64) if read is not None else 1.0) * xn[:, s] for s in range(S))
+    if row_idx is not None:
+        u = u[row_idx.long()]
+    return (u / torch.sqrt((u * u).mean(-1, keepdim=True) + eps) * weight.to(F64)).to(out_dtype)
+
+
+def scaled_sum_tensor(self):
+    return (self.sa * self.a.to(F64) + self.sb * self.b.to(F64)).to(torch.float32)
+
+
+# ---------------------------------------------------------------- attention with a soft cap
+def kv_store2(rows, k_off, v_off, row_pos, row_slot, kcache, vcache, page_table, page_size, ring, nkv, dk, dv):
+    for r in range(rows.shape[0]):
+        page, at = cache_offsets(page_table, int(row_slot[r]), int(row_pos[r]), page_size, ring)
+        kcache[page, :, at, :] = rows[r, k_off:k_off + nkv * dk].view(nkv, dk)
+        vcache[page, :, at, :] = rows[r, v_off:v_off + nkv * dv].view(nkv, dv)
+
+
+def _attend_capped(q, k, v, scale, cap):
+    """q [nh, dk], k [L, nkv, dk], v [L, nkv, dv]: every key visible."""
+    nh, per = q.shape[0], q.shape[0] // k.shape[1]
+    out = torch.zeros(nh, v.shape[2], dtype=F64)
+    for h in range(nh):
+        s = (k[:, h // per, :].to(F64) @ q[h].to(F64)) * scale
+        if cap:
+            s = cap * torch.tanh(s / cap)
+        out[h] = torch.softmax(s, dim=0) @ v[:, h // per, :].to(F64)
+    return out
+
+
+def _cached(kcache, vcache, page_table, slot, first, total, page_size, ring):
+    at = [cache_offsets(page_table, slot, pos, page_size, ring) for pos in range(first, total)]
+    return (torch.stack([kcache[p, :, r, :] for p, r in at]), torch.stack([vcache[p, :, r, :] for p, r in at]))
+
+
+def attn_cap_rows(q, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table, page_size, ring,
+                  n_seqs, max_rows, nh, nkv, dk, dv, scale, cap, window):
+    out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
+    for b in range(n_seqs):
+        s0, s1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
+        for a in range(s1 - s0):
+            pos = int(seq_start[b]) + a
+            first = max(0, pos - window + 1) if window and window > 0 else 0
+            k, v = _cached(kcache, vcache, page_table, int(seq_slot[b]), first, pos + 1, page_size, ring)
+            out[s0 + a] = _attend_capped(q[s0 + a, :nh * dk].view(nh, dk), k, v, scale, cap).reshape(-1).to(q.dtype)
+    return out
+
+
+def attn_cap_decode(q, kcache, vcache, page_table, page_size, ring, seq_slot, seq_len, nh, nkv, dk, dv,
+                    scale, cap, window, nsplit):
+    out = torch.zeros(q.shape[0], nh * dv, dtype=q.dtype)
+    for b in range(q.shape[0]):
+        n = int(seq_len[b])
+        first = max(0, n - window) if window and window > 0 else 0
+        k, v = _cached(kcache, vcache, page_table, int(seq_slot[b]), first, n, page_size, ring)
+        out[b] = _attend_capped(q[b, :nh * dk].view(nh, dk), k, v, scale, cap).reshape(-1).to(q.dtype)
+    return out
+
+
+# ---------------------------------------------------------------- the gated delta rule
+def delta_prepare(P, b_off, A, a_off, conv_w, tail, row_slot, a_log, dt_bias, G, H, dk, dv, per_channel):
+    T, C, taps = P.shape[0], conv_w.shape[0], conv_w.shape[1]
+    K, DW = taps - 1, dk if per_channel else 1
+    y = torch.zeros(T, C, dtype=F64)
+    for r in range(T):
+        slot, before = int(row_slot[r]), 0
+        while before < K and r - before - 1 >= 0 and int(row_slot[r - before - 1]) == slot:
+            before += 1
+        for j in range(taps):
+            d = K - j
+            src = P[r - d, :C] if d <= before else tail[slot, K - (d - before)]
+            y[r] += conv_w[:, j].to(F64) * src.to(F64)
+    y = y * torch.sigmoid(y)
+    unit = lambda x: x / torch.sqrt((x * x).sum(-1, keepdim=True) + 1e-6)
+    qn = unit(y[:, :G * dk].view(T, G, dk)) * dk ** -0.5
+    kn = unit(y[:, G * dk:2 * G * dk].view(T, G, dk))
+    vv = y[:, 2 * G * dk:].view(T, H, dv)
+    beta = torch.sigmoid(P[:, b_off:b_off + H].to(F64))
+    a = A[:, a_off:a_off + H * DW].to(F64) + dt_bias.to(F64)
+    sp = torch.where(a > 30, a, torch.log1p(torch.exp(torch.clamp(a, max=30))))
+    dec = torch.exp(-torch.exp(a_log.to(F64)).repeat_interleave(DW) * sp).view(T, H, DW)
+    return tuple(t.to(torch.float32).contiguous() for t in (qn, kn, vv, beta, dec))
+
+
+def delta_conv_tail(P, tail, cu_seqlens, seq_slot, n_seqs, taps):
+    K, C = taps - 1, tail.shape[2]
+    for b in range(n_seqs if K else 0):
+        r0, n, slot = int(cu_seqlens[b]), int(cu_seqlens[b + 1]) - int(cu_seqlens[b]), int(seq_slot[b])
+        if n <= 0:
+            continue
+        old = tail[slot].clone()
+        for j in range(K):
+            at = n - K + j
+            tail[slot, j] = P[r0 + at, :C].to(tail.dtype) if at >= 0 else old[j + n]
+
+
+def delta_scan(qn, kn, vv, beta, dec, state, cu_seqlens, seq_slot, n_seqs, max_rows):
+    T, G, dk = qn.shape
+    H, dv = vv.shape[1], vv.shape[2]
+    o = torch.zeros(T, H, dv, dtype=torch.float32)
+    for b in range(n_seqs):
+        slot = int(seq_slot[b])
+        for r in range(int(cu_seqlens[b]), int(cu_seqlens[b + 1])):
+            for h in range(H):
+                g = h // (H // G)
+                S = state[slot, h].to(F64) * dec[r, h].to(F64).expand(dk)[:, None]
+                u = beta[r, h].to(F64) * (vv[r, h].to(F64) - S.t() @ kn[r, g].to(F64))
+                S = S + torch.outer(kn[r, g].to(F64), u)
+                o[r, h] = (S.t() @ qn[r, g].to(F64)).to(torch.float32)
+                state[slot, h] = S.to(torch.float32)
+    return o
+
+
+def delta_finish(o, weight, Z, z_off, gate, eps, out_dtype):
+    T, H, dv = o.shape
+    z = Z[:, z_off:z_off + H * dv].to(F64).view(T, H, dv)
+    act = torch.sigmoid(z) if gate == "sigmoid" else z * torch.sigmoid(z)
+    x = o.to(F64)
+    return (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight.to(F64) * act).reshape(T, H * dv).to(out_dtype)
 
 
 def patch(monkeypatch):
@@ -409,5 +552,8 @@ def patch(monkeypatch):
                  "sum_rows", "relu_squared", "latent_rope_store", "latent_pack", "latent_gate",
                  "latent_decode_splits", "latent_decode_mfma_fits", "latent_attn_decode", "latent_absorb_q",
                  "latent_store_absorb",
-                 "few_outputs_f32", "moe_route", "moe_plan", "moe_experts", "moe_combine"):
+                 "few_outputs_f32", "moe_route", "moe_plan", "moe_experts", "moe_combine",
+                 "stream_mix_norm", "kv_store2", "attn_cap_rows", "attn_cap_decode", "delta_prepare",
+                 "delta_conv_tail", "delta_scan", "delta_finish"):
         monkeypatch.setattr(ops, name, globals()[name])
+    monkeypatch.setattr(ops.ScaledSum, "tensor", scaled_sum_tensor)
