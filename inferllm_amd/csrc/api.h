@@ -362,10 +362,11 @@ int illm_embed_streams(const int32_t* tokens, const void* table, int table_dt, f
 
 // ---- the gated delta rule (delta_rule.hip)
 int illm_delta_prepare(const void* P, int p_dt, int p_stride, int b_off, const void* A, int a_dt,
-                       int a_stride, int a_off, const float* conv_w, int taps, const void* tail,
+                       int a_stride, int a_off, const float* conv_w, int taps, void* tail,
                        int tail_dt, const int32_t* row_slot, const float* a_log,
                        const float* dt_bias, float* qn, float* kn, float* vv, float* beta,
-                       float* dec, int T, int G, int H, int dk, int dv, int DW, void* stream);
+                       float* dec, int T, int G, int H, int dk, int dv, int DW, int update_tail,
+                       void* stream);
 int illm_delta_conv_tail(const void* P, int p_dt, int p_stride, void* tail, int tail_dt,
                          const int32_t* cu, const int32_t* seq_slot, int n_seqs, int C, int taps,
                          void* stream);

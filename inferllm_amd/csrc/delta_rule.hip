@@ -22,51 +22,65 @@
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-// grid (rows); 256 threads; dynamic LDS: C floats.
+// grid (rows, NB); 256 threads.  A wave takes a head's vector at a time (q heads, k heads, v heads:
+// vector 4 y + w, then every 4 NB-th), lanes over its channels: convolution, SiLU, and for q and k the
+// unit norm, all in the wave.  beta and the decays are spread over all threads of the row's blocks.
 // P [T, p_stride]: columns [0, C) = q (G dk) | k (G dk) | v (H dv) before the convolution, b_off: H
 // columns of b.  A [T, a_stride] + a_off: the decays' pre-activations, DW a head (1 or dk).
+// `update_tail`: every sequence brings one row, and the lane that has read a channel's taps also
+// writes its tail for the next step (no other row reads that tail in this step).
+#define DELTA_VEC_MAX 4                                 // channels a lane holds: head sizes up to 256
 __global__ void __launch_bounds__(256)
 delta_prepare_kernel(const void* __restrict__ P, int p_dt, int p_stride, int b_off,
                      const void* __restrict__ A, int a_dt, int a_stride, int a_off,
-                     const float* __restrict__ conv_w, int taps, const void* __restrict__ tail,
+                     const float* __restrict__ conv_w, int taps, void* __restrict__ tail,
                      int tail_dt, const int32_t* __restrict__ row_slot,
                      const float* __restrict__ a_log, const float* __restrict__ dt_bias,
                      float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vv,
                      float* __restrict__ beta, float* __restrict__ dec, int G, int H, int dk, int dv,
-                     int DW) {
-    extern __shared__ float cs[];
-    const int r = blockIdx.x, tid = threadIdx.x;
+                     int DW, int update_tail) {
+    const int r = blockIdx.x, tid = threadIdx.x, NB = gridDim.y;
     const int C = 2 * G * dk + H * dv, K = taps - 1;
     const int slot = row_slot[r];
     int before = 0;                                     // rows of this sequence ahead of r in the step, up to K
     while (before < K && r - before - 1 >= 0 && row_slot[r - before - 1] == slot) ++before;
-    for (int c = tid; c < C; c += 256) {
-        float a = 0.f;
-        for (int j = 0; j < taps; ++j) {
-            const int d = K - j;                        // tap j looks d tokens back
-            float x;
-            if (d <= before) x = ld_f(P, p_dt, (size_t)(r - d) * p_stride + c);
-            else x = ld_f(tail, tail_dt, ((size_t)slot * K + (K - (d - before))) * C + c);
-            a = fmaf(conv_w[(size_t)c * taps + j], x, a);
-        }
-        cs[c] = a * sigmoid_f(a);
-    }
-    __syncthreads();
-    const int w = tid >> 6, lane = tid & 63;
+    const int w = wave_index(), lane = tid & 63;
     const float qscale = 1.0f / sqrtf((float)dk);
-    for (int vct = w; vct < 2 * G; vct += 4) {          // q heads, then k heads
-        const float* src = cs + (size_t)vct * dk;
+    for (int vct = blockIdx.y * 4 + w; vct < 2 * G + H; vct += 4 * NB) {
+        const bool is_v = vct >= 2 * G;
+        const int L = is_v ? dv : dk;
+        const int c0 = is_v ? 2 * G * dk + (vct - 2 * G) * dv : vct * dk;
+        float y[DELTA_VEC_MAX];
         float ss = 0.f;
-        for (int i = lane; i < dk; i += 64) ss += src[i] * src[i];
-        ss = wave_sum(ss);
-        const float inv = (vct < G ? qscale : 1.0f) / sqrtf(ss + 1e-6f);
-        float* dst = vct < G ? qn + ((size_t)r * G + vct) * dk : kn + ((size_t)r * G + (vct - G)) * dk;
-        for (int i = lane; i < dk; i += 64) dst[i] = src[i] * inv;
+#pragma unroll
+        for (int e = 0; e < DELTA_VEC_MAX; ++e) {
+            const int i = lane + 64 * e;
+            y[e] = 0.f;
+            if (i < L) {
+                const int c = c0 + i;
+                float a = 0.f, x = 0.f;
+                for (int j = 0; j < taps; ++j) {
+                    const int d = K - j;                // tap j looks d tokens back
+                    if (d <= before) x = ld_f(P, p_dt, (size_t)(r - d) * p_stride + c);
+                    else x = ld_f(tail, tail_dt, ((size_t)slot * K + (K - (d - before))) * C + c);
+                    a = fmaf(conv_w[(size_t)c * taps + j], x, a);
+                    if (update_tail && j > 0) st_f(tail, tail_dt, ((size_t)slot * K + (j - 1)) * C + c, x);
+                }
+                y[e] = a * sigmoid_f(a);
+                ss += y[e] * y[e];
+            }
+        }
+        float inv = 1.0f;
+        if (!is_v) inv = (vct < G ? qscale : 1.0f) / sqrtf(wave_sum(ss) + 1e-6f);
+        float* dst = is_v ? vv + ((size_t)r * H + (vct - 2 * G)) * dv
+                          : (vct < G ? qn + ((size_t)r * G + vct) * dk : kn + ((size_t)r * G + (vct - G)) * dk);
+#pragma unroll
+        for (int e = 0; e < DELTA_VEC_MAX; ++e)
+            if (lane + 64 * e < L) dst[lane + 64 * e] = y[e] * inv;
     }
-    for (int i = tid; i < H * dv; i += 256) vv[(size_t)r * H * dv + i] = cs[2 * G * dk + i];
-    for (int i = tid; i < H; i += 256)
+    for (int i = blockIdx.y * 256 + tid; i < H; i += 256 * NB)
         beta[(size_t)r * H + i] = sigmoid_f(ld_f(P, p_dt, (size_t)r * p_stride + b_off + i));
-    for (int i = tid; i < H * DW; i += 256) {
+    for (int i = blockIdx.y * 256 + tid; i < H * DW; i += 256 * NB) {
         const int hh = i / DW;
         const float a = ld_f(A, a_dt, (size_t)r * a_stride + a_off + i) + dt_bias[i];
         dec[(size_t)r * H * DW + i] = expf(-expf(a_log[hh]) * softplus_f(a));
@@ -75,24 +89,23 @@ delta_prepare_kernel(const void* __restrict__ P, int p_dt, int p_stride, int b_o
 
 extern "C" int illm_delta_prepare(const void* P, int p_dt, int p_stride, int b_off, const void* A,
                                   int a_dt, int a_stride, int a_off, const float* conv_w, int taps,
-                                  const void* tail, int tail_dt, const int32_t* row_slot,
+                                  void* tail, int tail_dt, const int32_t* row_slot,
                                   const float* a_log, const float* dt_bias, float* qn, float* kn,
                                   float* vv, float* beta, float* dec, int T, int G, int H, int dk,
-                                  int dv, int DW, void* stream) {
+                                  int dv, int DW, int update_tail, void* stream) {
     if (T < 0 || G <= 0 || H <= 0 || H % G || dk <= 0 || dv <= 0 || (DW != 1 && DW != dk) ||
+        dk > 64 * DELTA_VEC_MAX || dv > 64 * DELTA_VEC_MAX ||
         taps < 1 || taps > DELTA_MAX_TAPS || !illm_dtype_ok(p_dt) || !illm_dtype_ok(a_dt) ||
         !illm_dtype_ok(tail_dt))
         return ILLM_ERR_ARG;
-    const size_t C = 2 * (size_t)G * dk + (size_t)H * dv;
-    if (C * sizeof(float) > 150 * 1024) return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
-    if (C * sizeof(float) > 48 * 1024 &&
-        hipFuncSetAttribute((const void*)delta_prepare_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)(C * sizeof(float))) != hipSuccess)
-        return ILLM_ERR_LAUNCH;
-    hipLaunchKernelGGL(delta_prepare_kernel, dim3(T), dim3(256), C * sizeof(float), (hipStream_t)stream,
+    // blocks a row: enough to fill the chip when the rows are few
+    const int most = (2 * G + H + 3) / 4;
+    int nb = T >= 2048 ? 1 : (2048 + T - 1) / T;
+    nb = nb > most ? most : nb;
+    hipLaunchKernelGGL(delta_prepare_kernel, dim3(T, nb), dim3(256), 0, (hipStream_t)stream,
                        P, p_dt, p_stride, b_off, A, a_dt, a_stride, a_off, conv_w, taps, tail, tail_dt,
-                       row_slot, a_log, dt_bias, qn, kn, vv, beta, dec, G, H, dk, dv, DW);
+                       row_slot, a_log, dt_bias, qn, kn, vv, beta, dec, G, H, dk, dv, DW, update_tail);
     return illm_launch_status();
 }
 
@@ -141,7 +154,7 @@ extern "C" int illm_delta_conv_tail(const void* P, int p_dt, int p_stride, void*
 // asked for before this token's arithmetic.  state [slots][H][dk][dv] float32.
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 
 // The sum over the PARTS lanes of a group; every lane of the group gets the same bits.
@@ -156,77 +169,59 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
-template <int NS, int PARTS>
-__global__ void __launch_bounds__(64)
-delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
+// Steps of few tokens a sequence (single tokens above all): what counts is the state's bytes.
+// grid (ceil(dv / 64), H, sequences); 4 waves: a lane is a column, wave w holds rows [w NS, w NS + NS)
+// of it, so a row of S is read and written 256 bytes a wave; k, q and the decays of a row are the
+// same for a whole wave.  The waves' partial sums meet in LDS, in wave order.
+template <int NS>
+__global__ void __launch_bounds__(256)
+delta_step_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                   const float* __restrict__ vv, const float* __restrict__ beta,
                   const float* __restrict__ dec, int DW, float* __restrict__ state,
                   const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_slot,
                   float* __restrict__ o, int G, int H, int dk, int dv) {
-    constexpr int COLS = 64 / PARTS;
-    constexpr int NA = NS >= 4 ? 4 : NS;                // partial sums, to keep the chains short
-    const int b = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
-    const int part = lane % PARTS, col = blockIdx.x * COLS + lane / PARTS;
+    __shared__ float red[2][4][64];
+    const int b = blockIdx.z, h = blockIdx.y, lane = threadIdx.x & 63, w = wave_index();
+    const int col = blockIdx.x * 64 + lane;
     const int r0 = cu[b], n = cu[b + 1] - r0;
-    if (n <= 0) return;
-    const int slot = seq_slot[b], gh = h / (H / G), i0 = part * NS;
+    if (n <= 0) return;                                 // the whole block
+    const int slot = seq_slot[b], gh = h / (H / G), i0 = w * NS;
     const bool live = col < dv;
     float* sp = state + (((size_t)slot * H + h) * dk) * dv + col;
-    float s[NS], kc[NS], qc[NS], gc[NS];
+    float s[NS];
 #pragma unroll
     for (int ii = 0; ii < NS; ++ii) s[ii] = (live && i0 + ii < dk) ? sp[(size_t)(i0 + ii) * dv] : 0.f;
-    float vc, bc;
-#define DELTA_FETCH(ROW, K_, Q_, G_, V_, B_)                                                      \
-    {                                                                                             \
-        const float* kp = kn + ((size_t)(ROW) * G + gh) * dk;                                     \
-        const float* qp = qn + ((size_t)(ROW) * G + gh) * dk;                                     \
-        const float* dp = dec + ((size_t)(ROW) * H + h) * DW;                                     \
-        _Pragma("unroll") for (int ii = 0; ii < NS; ++ii) {                                       \
-            const int i = i0 + ii;                                                                \
-            const bool in = i < dk;                                                               \
-            K_[ii] = in ? kp[i] : 0.f;                                                            \
-            Q_[ii] = in ? qp[i] : 0.f;                                                            \
-            G_[ii] = in ? (DW == 1 ? dp[0] : dp[i]) : 1.f;                                        \
-        }                                                                                         \
-        V_ = live ? vv[((size_t)(ROW) * H + h) * dv + col] : 0.f;                                 \
-        B_ = beta[(size_t)(ROW) * H + h];                                                         \
-    }
-    DELTA_FETCH(r0, kc, qc, gc, vc, bc)
     for (int t = 0; t < n; ++t) {
         const int row = r0 + t;
-        float kx[NS], qx[NS], gx[NS], vx, bx;
-        const int nxt = t + 1 < n ? row + 1 : row;
-        DELTA_FETCH(nxt, kx, qx, gx, vx, bx)
-        float pa[NA];
-#pragma unroll
-        for (int a = 0; a < NA; ++a) pa[a] = 0.f;
+        const float* kp = kn + ((size_t)row * G + gh) * dk;
+        const float* qp = qn + ((size_t)row * G + gh) * dk;
+        const float* dp = dec + ((size_t)row * H + h) * DW;
+        float kc[NS], pa[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ii = 0; ii < NS; ++ii) {
-            s[ii] *= gc[ii];
-            pa[ii % NA] = fmaf(s[ii], kc[ii], pa[ii % NA]);
+            const int i = i0 + ii;
+            kc[ii] = i < dk ? kp[i] : 0.f;
+            s[ii] *= i < dk ? (DW == 1 ? dp[0] : dp[i]) : 1.f;
+            pa[ii & 3] = fmaf(s[ii], kc[ii], pa[ii & 3]);
         }
-        float kv = pa[0];
-#pragma unroll
-        for (int a = 1; a < NA; ++a) kv += pa[a];
-        kv = group_sum<PARTS>(kv);
-        const float u = bc * (vc - kv);
-#pragma unroll
-        for (int a = 0; a < NA; ++a) pa[a] = 0.f;
+        red[0][w][lane] = (pa[0] + pa[1]) + (pa[2] + pa[3]);
+        __syncthreads();
+        const float kv = (red[0][0][lane] + red[0][1][lane]) + (red[0][2][lane] + red[0][3][lane]);
+        const float v = live ? vv[((size_t)row * H + h) * dv + col] : 0.f;
+        const float u = beta[(size_t)row * H + h] * (v - kv);
+        pa[0] = pa[1] = pa[2] = pa[3] = 0.f;
 #pragma unroll
         for (int ii = 0; ii < NS; ++ii) {
+            const int i = i0 + ii;
             s[ii] = fmaf(kc[ii], u, s[ii]);
-            pa[ii % NA] = fmaf(s[ii], qc[ii], pa[ii % NA]);
+            pa[ii & 3] = fmaf(s[ii], i < dk ? qp[i] : 0.f, pa[ii & 3]);
         }
-        float ov = pa[0];
-#pragma unroll
-        for (int a = 1; a < NA; ++a) ov += pa[a];
-        ov = group_sum<PARTS>(ov);
-        if (part == 0 && live) o[((size_t)row * H + h) * dv + col] = ov;
-#pragma unroll
-        for (int ii = 0; ii < NS; ++ii) { kc[ii] = kx[ii]; qc[ii] = qx[ii]; gc[ii] = gx[ii]; }
-        vc = vx; bc = bx;
+        red[1][w][lane] = (pa[0] + pa[1]) + (pa[2] + pa[3]);
+        __syncthreads();
+        if (w == 0 && live)
+            o[((size_t)row * H + h) * dv + col] =
+                (red[1][0][lane] + red[1][1][lane]) + (red[1][2][lane] + red[1][3][lane]);
     }
-#undef DELTA_FETCH
 #pragma unroll
     for (int ii = 0; ii < NS; ++ii)
         if (live && i0 + ii < dk) sp[(size_t)(i0 + ii) * dv] = s[ii];
@@ -236,7 +231,7 @@ delta_scan_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
 // dependent operations a token, so nothing may wait for memory inside it: the k, q and decay rows of
 // DELTA_CHUNK tokens go through LDS in two buffers, the next chunk's loads (and its v and beta, in
 // registers) are issued before this chunk's arithmetic and stored after it.  One wave a block;
-// dynamic LDS: 2 * DELTA_CHUNK * (2 dk + DW) floats.
+// dynamic LDS: 2 * DELTA_CHUNK * 3 * 16 NS floats.
 #define DELTA_CHUNK 8
 template <int NS>
 __global__ void __launch_bounds__(64)
@@ -246,44 +241,48 @@ delta_scan_long_kernel(const float* __restrict__ qn, const float* __restrict__ k
                        const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_slot,
                        float* __restrict__ o, int G, int H, int dk, int dv) {
     constexpr int PARTS = 16, COLS = 4, TC = DELTA_CHUNK;
-    constexpr int JJ = NS >= 4 ? NS / 4 : 1;            // pieces of 64 floats in a row of 16 NS
+    constexpr int DKP = PARTS * NS;                     // a row of k, q or decays in LDS, filled up
+    constexpr int JJ = (DKP + 63) / 64;                 // pieces of 64 floats in it
     constexpr int NA = NS >= 4 ? 4 : NS;
-    extern __shared__ float stage[];
+    extern __shared__ float stage[];                    // [2][TC][k | q | decay][DKP]
     const int b = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
     const int part = lane % PARTS, col = blockIdx.x * COLS + lane / PARTS;
     const int r0 = cu[b], n = cu[b + 1] - r0;
     if (n <= 0) return;
     const int slot = seq_slot[b], gh = h / (H / G);
     const bool live = col < dv;
-    const int RW = 2 * dk + DW;
     float* sp = state + (((size_t)slot * H + h) * dk) * dv + col;
     float s[NS];
 #pragma unroll
     for (int ii = 0; ii < NS; ++ii)      // row part + 16 ii: the 16 parts read neighbouring words of LDS
         s[ii] = (live && part + PARTS * ii < dk) ? sp[(size_t)(part + PARTS * ii) * dv] : 0.f;
+    const float* kbase = kn + ((size_t)r0 * G + gh) * dk;
+    const float* qbase = qn + ((size_t)r0 * G + gh) * dk;
+    const float* dbase = dec + ((size_t)r0 * H + h) * DW;
+    const float* vbase = vv + ((size_t)r0 * H + h) * dv + (live ? col : 0);
+    const float* bbase = beta + (size_t)r0 * H + h;
+    float* op = o + ((size_t)r0 * H + h) * dv + col;
+    const int kstep = G * dk, dstep = H * DW, vstep = H * dv;
     float sk[TC][JJ], sq[TC][JJ], sg[TC][JJ], sv[TC], sb[TC];
+    // rows beyond dk are filled with k = q = 0 and decay 1, so the arithmetic needs no bounds
 #define DELTA_LOAD(T0)                                                                            \
     _Pragma("unroll") for (int tt = 0; tt < TC; ++tt) {                                           \
-        const int row = r0 + ((T0) + tt < n ? (T0) + tt : n - 1);                                 \
-        const float* kp = kn + ((size_t)row * G + gh) * dk;                                       \
-        const float* qp = qn + ((size_t)row * G + gh) * dk;                                       \
-        const float* dp = dec + ((size_t)row * H + h) * DW;                                       \
+        const int at = (T0) + tt < n ? (T0) + tt : n - 1;                                         \
         _Pragma("unroll") for (int jj = 0; jj < JJ; ++jj) {                                       \
             const int j = lane + 64 * jj;                                                         \
-            sk[tt][jj] = j < dk ? kp[j] : 0.f;                                                    \
-            sq[tt][jj] = j < dk ? qp[j] : 0.f;                                                    \
-            sg[tt][jj] = j < DW ? dp[j] : 1.f;                                                    \
+            sk[tt][jj] = j < dk ? kbase[(size_t)at * kstep + j] : 0.f;                            \
+            sq[tt][jj] = j < dk ? qbase[(size_t)at * kstep + j] : 0.f;                            \
+            sg[tt][jj] = j < dk ? dbase[(size_t)at * dstep + (DW == 1 ? 0 : j)] : 1.f;            \
         }                                                                                         \
-        sv[tt] = live ? vv[((size_t)row * H + h) * dv + col] : 0.f;                               \
-        sb[tt] = beta[(size_t)row * H + h];                                                       \
+        sv[tt] = vbase[(size_t)at * vstep];                                                       \
+        sb[tt] = bbase[(size_t)at * H];                                                           \
     }
 #define DELTA_STORE(BUF)                                                                          \
     _Pragma("unroll") for (int tt = 0; tt < TC; ++tt) {                                           \
-        float* dst = stage + ((size_t)(BUF) * TC + tt) * RW;                                      \
+        float* dst = stage + ((size_t)(BUF) * TC + tt) * 3 * DKP;                                 \
         _Pragma("unroll") for (int jj = 0; jj < JJ; ++jj) {                                       \
             const int j = lane + 64 * jj;                                                         \
-            if (j < dk) { dst[j] = sk[tt][jj]; dst[dk + j] = sq[tt][jj]; }                        \
-            if (j < DW) dst[2 * dk + j] = sg[tt][jj];                                             \
+            if (j < DKP) { dst[j] = sk[tt][jj]; dst[DKP + j] = sq[tt][jj]; dst[2 * DKP + j] = sg[tt][jj]; } \
         }                                                                                         \
     }
     DELTA_LOAD(0)
@@ -295,25 +294,18 @@ delta_scan_long_kernel(const float* __restrict__ qn, const float* __restrict__ k
         for (int tt = 0; tt < TC; ++tt) { cv[tt] = sv[tt]; cb[tt] = sb[tt]; }
         const bool more = t0 + TC < n;
         if (more) DELTA_LOAD(t0 + TC)
+        const float* src0 = stage + (size_t)buf * TC * 3 * DKP + part;
 #pragma unroll
         for (int tt = 0; tt < TC; ++tt) {
             if (t0 + tt < n) {
-                const float* src = stage + ((size_t)buf * TC + tt) * RW;
-                float kc[NS], qc[NS], gc[NS];
-#pragma unroll
-                for (int ii = 0; ii < NS; ++ii) {
-                    const int i = part + PARTS * ii;
-                    const bool in = i < dk;
-                    kc[ii] = in ? src[i] : 0.f;
-                    qc[ii] = in ? src[dk + i] : 0.f;
-                    gc[ii] = in ? src[2 * dk + (DW == 1 ? 0 : i)] : 1.f;
-                }
-                float pa[NA];
+                const float* src = src0 + tt * 3 * DKP;
+                float kc[NS], pa[NA];
 #pragma unroll
                 for (int a = 0; a < NA; ++a) pa[a] = 0.f;
 #pragma unroll
                 for (int ii = 0; ii < NS; ++ii) {
-                    s[ii] *= gc[ii];
+                    kc[ii] = src[PARTS * ii];
+                    s[ii] *= src[2 * DKP + PARTS * ii];
                     pa[ii % NA] = fmaf(s[ii], kc[ii], pa[ii % NA]);
                 }
                 float kv = pa[0];
@@ -326,13 +318,14 @@ delta_scan_long_kernel(const float* __restrict__ qn, const float* __restrict__ k
 #pragma unroll
                 for (int ii = 0; ii < NS; ++ii) {
                     s[ii] = fmaf(kc[ii], u, s[ii]);
-                    pa[ii % NA] = fmaf(s[ii], qc[ii], pa[ii % NA]);
+                    pa[ii % NA] = fmaf(s[ii], src[DKP + PARTS * ii], pa[ii % NA]);
                 }
                 float ov = pa[0];
 #pragma unroll
                 for (int a = 1; a < NA; ++a) ov += pa[a];
                 ov = group_sum<PARTS>(ov);
-                if (part == 0 && live) o[((size_t)(r0 + t0 + tt) * H + h) * dv + col] = ov;
+                if (part == 0 && live) *op = ov;
+                op += vstep;
             }
         }
         if (more) DELTA_STORE(buf ^ 1)
@@ -357,12 +350,9 @@ extern "C" int illm_delta_scan(const float* qn, const float* kn, const float* vv
         return ILLM_ERR_ARG;
     if (n_seqs == 0) return ILLM_OK;
     hipStream_t st = (hipStream_t)stream;
-#define GO(NS_, PARTS_)                                                                          \
-    hipLaunchKernelGGL((delta_scan_kernel<NS_, PARTS_>), dim3((dv + 64 / PARTS_ - 1) / (64 / PARTS_), H, n_seqs), \
-                       dim3(64), 0, st, qn, kn, vv, beta, dec, DW, state, cu, seq_slot, o, G, H, dk, dv)
     if (max_rows >= 16) {
         const int ns = (dk + 15) / 16;
-        const size_t lds = (size_t)2 * DELTA_CHUNK * (2 * dk + DW) * sizeof(float);
+        const size_t lds = (size_t)2 * DELTA_CHUNK * 3 * 16 * (ns <= 1 ? 1 : ns <= 2 ? 2 : ns <= 4 ? 4 : ns <= 8 ? 8 : 16) * sizeof(float);
         const dim3 grid((dv + 3) / 4, H, n_seqs);
 #define GOL(NS_)                                                                                  \
     hipLaunchKernelGGL(delta_scan_long_kernel<NS_>, grid, dim3(64), lds, st, qn, kn, vv, beta, dec, DW, \
@@ -375,13 +365,17 @@ extern "C" int illm_delta_scan(const float* qn, const float* kn, const float* vv
 #undef GOL
     } else {
         const int ns = (dk + 3) / 4;
-        if (ns <= 4) GO(4, 4);
-        else if (ns <= 8) GO(8, 4);
-        else if (ns <= 16) GO(16, 4);
-        else if (ns <= 32) GO(32, 4);
-        else GO(64, 4);
+        const dim3 grid((dv + 63) / 64, H, n_seqs);
+#define GOS(NS_)                                                                                  \
+    hipLaunchKernelGGL(delta_step_kernel<NS_>, grid, dim3(256), 0, st, qn, kn, vv, beta, dec, DW, state, \
+                       cu, seq_slot, o, G, H, dk, dv)
+        if (ns <= 4) GOS(4);
+        else if (ns <= 8) GOS(8);
+        else if (ns <= 16) GOS(16);
+        else if (ns <= 32) GOS(32);
+        else GOS(64);
+#undef GOS
     }
-#undef GO
     return illm_launch_status();
 }
 

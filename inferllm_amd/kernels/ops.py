@@ -1494,14 +1494,16 @@ def attn_cap_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
 # ------------------------------------------------------------------ the gated delta rule
 def delta_prepare(P: torch.Tensor, b_off: int, A: torch.Tensor, a_off: int, conv_w: torch.Tensor,
                   tail: torch.Tensor, row_slot: torch.Tensor, a_log: torch.Tensor,
-                  dt_bias: torch.Tensor, G: int, H: int, dk: int, dv: int, per_channel: bool):
+                  dt_bias: torch.Tensor, G: int, H: int, dk: int, dv: int, per_channel: bool,
+                  update_tail: bool = False):
     """From the projections P [T, n] = [q (G dk) | k (G dk) | v (H dv) | ...] the recurrence's
     float32 inputs: q and k after the short convolution (conv_w float32 [C, taps], the inputs
     before a step's first row from `tail` [slots, taps - 1, C]), SiLU and the unit norm per head
     (q also times dk^-1/2), v after convolution and SiLU, beta = sigmoid(P[:, b_off + h]) and the
     decays exp(-exp(a_log[h]) softplus(A[:, a_off + i] + dt_bias[i])), one a head or, with
-    `per_channel`, one a head and key channel.  Returns (q [T, G, dk], k, v [T, H, dv],
-    beta [T, H], decay [T, H, 1 or dk])."""
+    `per_channel`, one a head and key channel.  `update_tail` (every sequence brings exactly one
+    row): the tail is also moved on by that row here, and `delta_conv_tail` is not needed.
+    Returns (q [T, G, dk], k, v [T, H, dv], beta [T, H], decay [T, H, 1 or dk])."""
     _gpu(P, A, conv_w, tail, row_slot, a_log, dt_bias)
     T = P.shape[0]
     _i32(row_slot, T)
@@ -1524,7 +1526,7 @@ def delta_prepare(P: torch.Tensor, b_off: int, A: torch.Tensor, a_off: int, conv
     _check(_lib().illm_delta_prepare(
         _p(P), _code(P), P.shape[1], b_off, _p(A), _code(A), A.shape[1], a_off, _p(conv_w), taps,
         _p(tail), _code(tail), _p(row_slot), _p(a_log), _p(dt_bias), _p(qn), _p(kn), _p(vv), _p(beta),
-        _p(dec), T, G, H, dk, dv, DW, _stream()), "delta_prepare")
+        _p(dec), T, G, H, dk, dv, DW, 1 if update_tail else 0, _stream()), "delta_prepare")
     return qn, kn, vv, beta, dec
 
 

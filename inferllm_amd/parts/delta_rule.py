@@ -46,8 +46,8 @@ class GatedDeltaRule(Mixer):
             raise ValueError(f"gated delta rule: decay {decay!r} or gate {gate!r} is unknown")
         if not 1 <= int(conv) <= 8:
             raise ValueError(f"gated delta rule: {conv} taps; the kernels take 1 to 8")
-        if key_dim > 256:
-            raise ValueError(f"gated delta rule: key_dim {key_dim} is beyond the kernels' limit of 256")
+        if key_dim > 256 or value_dim > 256:
+            raise ValueError(f"gated delta rule: head sizes {key_dim}, {value_dim} are beyond the kernels' limit of 256")
         self.E, self.H, self.G = int(hidden_size), int(num_heads), int(num_kv_heads)
         self.dk, self.dv, self.taps, self.eps = int(key_dim), int(value_dim), int(conv), float(eps)
         self.per_channel, self.gate = decay == "channel", gate
@@ -121,8 +121,10 @@ class GatedDeltaRule(Mixer):
         S, tail = state["S"], state["tail"]
         qn, kn, vv, beta, dec = ops.delta_prepare(
             P, self.b_off, P2 if self.ra else P, self.a_off, self.conv_w, tail, ctx.row_slot,
-            self.a_log, self.dt_bias, self.G, self.H, self.dk, self.dv, self.per_channel)
-        ops.delta_conv_tail(P, tail, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs, self.taps)
+            self.a_log, self.dt_bias, self.G, self.H, self.dk, self.dv, self.per_channel,
+            update_tail=not ctx.prefill)
+        if ctx.prefill:
+            ops.delta_conv_tail(P, tail, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs, self.taps)
         o = ops.delta_scan(qn, kn, vv, beta, dec, S, ctx.cu_seqlens, ctx.seq_slot, ctx.n_seqs,
                            ctx.max_rows if ctx.prefill else 1)
         y = ops.delta_finish(o, self.norm_w, P2 if self.rg else P, self.z_off, self.gate, self.eps,

@@ -482,7 +482,8 @@ def attn_cap_decode(q, kcache, vcache, page_table, page_size, ring, seq_slot, se
 
 
 # ---------------------------------------------------------------- the gated delta rule
-def delta_prepare(P, b_off, A, a_off, conv_w, tail, row_slot, a_log, dt_bias, G, H, dk, dv, per_channel):
+def delta_prepare(P, b_off, A, a_off, conv_w, tail, row_slot, a_log, dt_bias, G, H, dk, dv, per_channel,
+                  update_tail=False):
     T, C, taps = P.shape[0], conv_w.shape[0], conv_w.shape[1]
     K, DW = taps - 1, dk if per_channel else 1
     y = torch.zeros(T, C, dtype=F64)
@@ -503,6 +504,10 @@ def delta_prepare(P, b_off, A, a_off, conv_w, tail, row_slot, a_log, dt_bias, G,
     a = A[:, a_off:a_off + H * DW].to(F64) + dt_bias.to(F64)
     sp = torch.where(a > 30, a, torch.log1p(torch.exp(torch.clamp(a, max=30))))
     dec = torch.exp(-torch.exp(a_log.to(F64)).repeat_interleave(DW) * sp).view(T, H, DW)
+    if update_tail:                                   # one row a sequence: its tail moves on by that row
+        for r in range(T if K else 0):
+            slot = int(row_slot[r])
+            tail[slot] = torch.cat([tail[slot, 1:], P[r:r + 1, :C].to(tail.dtype)])
     return tuple(t.to(torch.float32).contiguous() for t in (qn, kn, vv, beta, dec))
 
 
