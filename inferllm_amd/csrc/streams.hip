@@ -12,8 +12,19 @@
 
 #define STREAMS_MAX 8
 
-// grid (rows); dynamic LDS: E floats (u) + 16.
-template <int S>
+__device__ __forceinline__ void ld4(const void* p, int dt, size_t i, float* o) {
+    if (dt == ILLM_BF16) {
+        const uint2 u = *(const uint2*)((const bf16_t*)p + i);
+        o[0] = __uint_as_float(u.x << 16); o[1] = __uint_as_float(u.x & 0xffff0000u);
+        o[2] = __uint_as_float(u.y << 16); o[3] = __uint_as_float(u.y & 0xffff0000u);
+    } else {
+        const float4 f = *(const float4*)((const float*)p + i);
+        o[0] = f.x; o[1] = f.y; o[2] = f.z; o[3] = f.w;
+    }
+}
+
+// grid (rows); dynamic LDS: E floats (u) + 16.  VEC: E is a multiple of 4.
+template <int S, bool VEC>
 __global__ void __launch_bounds__(256)
 stream_mix_norm_kernel(float* __restrict__ x, const void* __restrict__ y1, int y1_dt, float ya,
                        const void* __restrict__ y2, int y2_dt, float yb,
@@ -36,6 +47,52 @@ stream_mix_norm_kernel(float* __restrict__ x, const void* __restrict__ y1, int y
         for (int t = 0; t < S; ++t) m[s][t] = y1 ? mix[s * S + t] : (s == t ? 1.f : 0.f);
     }
     float ss = 0.f;
+    if (VEC) {
+        // four neighbouring columns a thread: 16-byte loads and stores of every stream
+        for (int i = threadIdx.x * 4; i < E; i += 1024) {
+            float4 xs[S];
+            float xn[S][4];
+#pragma unroll
+            for (int s = 0; s < S; ++s) xs[s] = *(const float4*)(xr + (size_t)s * E + i);
+            if (y1) {
+                float y[4];
+                ld4(y1, y1_dt, row * E + i, y);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) y[c] *= ya;
+                if (y2) {
+                    float z[4];
+                    ld4(y2, y2_dt, row * E + i, z);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) y[c] += yb * z[c];
+                }
+#pragma unroll
+                for (int t = 0; t < S; ++t) {
+                    float a[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s = 0; s < S; ++s) {
+                        a[0] += m[s][t] * xs[s].x; a[1] += m[s][t] * xs[s].y;
+                        a[2] += m[s][t] * xs[s].z; a[3] += m[s][t] * xs[s].w;
+                    }
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) xn[t][c] = a[c] + ow[t] * y[c];
+                    if (!row_idx)
+                        *(float4*)(xr + (size_t)t * E + i) = make_float4(xn[t][0], xn[t][1], xn[t][2], xn[t][3]);
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < S; ++t) {
+                    xn[t][0] = xs[t].x; xn[t][1] = xs[t].y; xn[t][2] = xs[t].z; xn[t][3] = xs[t].w;
+                }
+            }
+            float u[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < S; ++s)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) u[c] += rd[s] * xn[s][c];
+            *(float4*)(us + i) = make_float4(u[0], u[1], u[2], u[3]);
+            ss += u[0] * u[0]; ss += u[1] * u[1]; ss += u[2] * u[2]; ss += u[3] * u[3];
+        }
+    } else
     for (int i = threadIdx.x; i < E; i += 256) {
         float xs[S], xn[S];
 #pragma unroll
@@ -82,19 +139,24 @@ extern "C" int illm_stream_mix_norm(float* x, int S, const void* y1, int y1_dt, 
     if (rows == 0) return ILLM_OK;
     const size_t lds = ((size_t)E + 16) * sizeof(float);
     hipStream_t st = (hipStream_t)stream;
-#define GO(S_)                                                                                    \
-    case S_:                                                                                      \
+#define GO1(S_, V_)                                                                               \
+    {                                                                                             \
         if (lds > 48 * 1024 &&                                                                    \
-            hipFuncSetAttribute((const void*)stream_mix_norm_kernel<S_>,                          \
+            hipFuncSetAttribute((const void*)stream_mix_norm_kernel<S_, V_>,                      \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
             return ILLM_ERR_LAUNCH;                                                               \
-        hipLaunchKernelGGL(stream_mix_norm_kernel<S_>, dim3(rows), dim3(256), lds, st, x, y1, y1_dt, \
+        hipLaunchKernelGGL((stream_mix_norm_kernel<S_, V_>), dim3(rows), dim3(256), lds, st, x, y1, y1_dt, \
                            ya, y2, y2_dt, yb, mix, outw, read, w, w_dt, h, h_dt, row_idx, E, eps); \
+    }
+#define GO(S_)                                                                                    \
+    case S_:                                                                                      \
+        if (E % 4 == 0) GO1(S_, true) else GO1(S_, false)                                         \
         break;
     switch (S) {
         GO(1) GO(2) GO(3) GO(4) GO(5) GO(6) GO(7) GO(8)
     }
 #undef GO
+#undef GO1
     return illm_launch_status();
 }
 

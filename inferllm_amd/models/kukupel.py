@@ -71,6 +71,8 @@ class KukupelConfig:
     streams: int = 0                      # 0: one residual stream, plain pre-norm layers
     layers: List[dict] = field(default_factory=list)
     max_positions: int = DEFAULT_MAX_POSITIONS
+    unused_tensors: List[str] = field(default_factory=list)    # in the folder, without a part to act on
+    mix_without_ff: List[int] = field(default_factory=list)    # layers without feed-forward that still mix
 
     architecture = "Kukupel"
     cli_type_names = ("kukupel",)
@@ -144,6 +146,14 @@ class KukupelConfig:
         -> shape), where the configuration does not state them."""
         cfg = copy.deepcopy(self)
         for i, layer in enumerate(cfg.layers):
+            if layer.get("mlp") is None:
+                # a layer without a feed-forward whose folder still holds the second sublayer's
+                # tensors: its norm and its read and output weights have nothing to act on (they are
+                # left in the file), its mix matrix still mixes the streams
+                cfg.unused_tensors += [n for n in (f"l{i}.norm2", f"l{i}.hc2.in", f"l{i}.hc2.out") if n in shapes]
+                if f"l{i}.hc2.mix" in shapes:
+                    (cfg.mix_without_ff if self.streams else cfg.unused_tensors).append(
+                        i if self.streams else f"l{i}.hc2.mix")
             if layer.get("type") != "parallel":
                 continue
             right = layer["mixer"]["right"]
@@ -213,6 +223,8 @@ class KukupelConfig:
             if S:
                 for q in (1, 2) if has_ff else (1,):
                     block_tensors.update({f"mix{q}": f"l{i}.hc{q}.mix", f"out{q}": f"l{i}.hc{q}.out"})
+                if i in self.mix_without_ff:
+                    block_tensors["mix2"] = f"l{i}.hc2.mix"
             layers.append(LayerSpec(
                 block="hyper_connections" if S else "pre_norm",
                 mixer=self._mixer(i, layer),
@@ -231,4 +243,4 @@ class KukupelConfig:
             schedule=[ScheduleEntry(layer=i, cache_line=i) for i in range(len(layers))],
             final_norm=norm("final.norm"),
             head=PartSpec("lm_head", {"hidden_size": E, "vocab_size": V}, {"weight": "embed"}),
-            bos_token_id=None, eos_token_ids=[])
+            bos_token_id=None, eos_token_ids=[], ignored_tensor_suffixes=list(self.unused_tensors))

@@ -88,7 +88,10 @@ class HyperConnectionBlock(Block):
     The reads belong to the norms (`stream_rms_norm`, whose kernel also does the write of the
     sublayer before it); the block owns mix_q [streams, streams] (indexed [from, to]) and out_q
     [streams] and hands each sublayer's output on as `ops.StreamWrite`, the last one to whatever
-    norm comes next.  A layer whose feed-forward is "none" has the mixer's sublayer alone.
+    norm comes next.  A layer whose feed-forward is "none" has the mixer's sublayer alone; if it is
+    given the second sublayer's mix matrix all the same (`mix2` among its tensors), the streams are
+    still mixed by it, with nothing added: folded at load into the first sublayer's write,
+    x <- M2^T (M1^T x + out1 y) = (M1 M2)^T x + (M2^T out1) y.
     """
 
     graph_safe_prompts = True
@@ -108,12 +111,18 @@ class HyperConnectionBlock(Block):
         mix = lambda: TensorWant((S, S), init="eye_normal", keep_stored=True)
         out = lambda: TensorWant((S,), init="ones_normal", keep_stored=True)
         out = {"mix1": mix(), "out1": out()} | ({"mix2": mix(), "out2": out()} if self.has_ff else {})
+        if not self.has_ff and "mix2" in self.tensors:
+            out["mix2"] = mix()
         return out
 
     def load_own(self, tensors) -> None:
         for q in range(2 if self.has_ff else 1):
             self.mix[q] = self._take(tensors, f"mix{q + 1}").to(torch.float32).contiguous()
             self.out[q] = self._take(tensors, f"out{q + 1}").to(torch.float32).contiguous()
+        if not self.has_ff and "mix2" in self.tensors:
+            second = self._take(tensors, "mix2").to(torch.float32)
+            self.out[0] = (self.out[0] @ second).contiguous()
+            self.mix[0] = (self.mix[0] @ second).contiguous()
 
     def _write(self, y, q: int) -> ops.StreamWrite:
         if isinstance(y, ops.ScaledSum):

@@ -132,9 +132,11 @@ def forward(config, w, tokens, layers_out=None, margins=None):
     xs = [x.clone() for _ in range(max(S, 1))]
     for i, layer in enumerate(config["layers"]):
         for q in (1, 2):
-            if q == 2 and layer.get("mlp") is None:
-                continue
             hc = f"l{i}.hc{q}."
+            if q == 2 and layer.get("mlp") is None:
+                if S and hc + "mix" in w:        # no sublayer, but a mix matrix: the streams are still mixed
+                    xs = [sum(w[hc + "mix"][s, t] * xs[s] for s in range(S)) for t in range(S)]
+                continue
             u = sum(w[hc + "in"][s] * xs[s] for s in range(S)) if S else xs[0]
             hn = rms_norm(u, w[f"l{i}.norm{q}"], eps)
             y = mixer(hn, w, i, layer, eps) if q == 1 else experts(hn, w, f"l{i}.mlp.", layer["mlp"], margins)

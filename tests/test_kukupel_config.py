@@ -119,3 +119,17 @@ def test_plain_convolution_sees_only_the_past():
     silu = lambda z: z * torch.sigmoid(z)
     assert torch.equal(y[:3], torch.zeros(3, 2, dtype=torch.float64)) and torch.equal(y[6], torch.zeros(2, dtype=torch.float64))
     assert torch.allclose(y[3], silu(w[:, 2])) and torch.allclose(y[4], silu(w[:, 1])) and torch.allclose(y[5], silu(w[:, 0]))
+
+
+def test_a_layer_without_feed_forward_tolerates_the_second_sublayers_tensors():
+    """A folder may hold norm2 and hc2.* of a layer whose mlp is null: nothing acts on the norm and
+    the read and output weights; the mix matrix, if there, still mixes the streams."""
+    import inferllm_amd as I
+    from inferllm_amd.engine.model import expected_tensors
+    shapes = {"l2.norm2": (96,), "l2.hc2.in": (2,), "l2.hc2.out": (2,), "l2.hc2.mix": (2, 2)}
+    cfg = I.config_from_dict(MIXED).with_tensor_shapes(shapes)
+    spec = cfg.to_spec()
+    want = expected_tensors(spec)
+    assert want["l2.hc2.mix"].shape == (2, 2) and "l2.hc2.in" not in want and "l2.norm2" not in want
+    assert sorted(spec.ignored_tensor_suffixes) == ["l2.hc2.in", "l2.hc2.out", "l2.norm2"]
+    assert "l2.hc2.mix" not in expected_tensors(I.config_from_dict(MIXED).to_spec())

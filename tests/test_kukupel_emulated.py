@@ -60,3 +60,31 @@ def test_prompts_tokens_and_portions_equal_plain(name, tmp_path, emulated):
     assert (torch.cat(rows).double() - plain[0]).abs().max() < 1e-4
     r.cache.free_slot(s)
     r.cache.check()
+
+
+def test_a_mix_matrix_without_its_sublayer_still_mixes(tmp_path, emulated):
+    """A layer without feed-forward whose folder holds the second sublayer's tensors."""
+    config = NO_KEYS
+    g = torch.Generator().manual_seed(4)
+
+    def edit(w):
+        w["l1.hc2.mix"] = torch.eye(3, dtype=torch.float64) + 0.3 * torch.randn(3, 3, generator=g, dtype=torch.float64)
+        w["l1.hc2.in"] = torch.ones(3, dtype=torch.float64)
+        w["l1.norm2"] = torch.ones(48, dtype=torch.float64)
+    d = write_model(tmp_path, config, seed=5, edit=edit)
+    w = weights64(d)
+    from inferllm_amd.weights.loader import stored_shapes
+    cfg = I.config_from_dict(config).with_tensor_shapes(stored_shapes(d))
+    model = DecoderModel(cfg.to_spec())
+    assert "l1.hc2.mix" in model.wants() and "l1.norm2" not in model.wants()
+    model.load({k: v.to(torch.float32) for k, v in w.items() if k in model.wants()})
+    cache = CacheManager(model.kv_lines(), model.state_lines(), max_tokens=256, max_slots=2,
+                         max_seq_len=128, dtype=torch.float32, device="cpu")
+    r = StepRunner(model, cache, torch.float32, torch.device("cpu"), use_graphs=False)
+    ids = random_ids(20, config["vocab"], 8)
+    s = cache.alloc_slot()
+    out = r.step([StepEntry(s, ids, list(range(20)))])
+    assert (out.double() - P.forward(config, w, ids)).abs().max() < 1e-4
+    plain = dict(w)
+    del plain["l1.hc2.mix"]
+    assert (P.forward(config, plain, ids) - P.forward(config, w, ids)).abs().max() > 1e-3
