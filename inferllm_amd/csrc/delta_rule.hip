@@ -264,18 +264,47 @@ delta_scan_long_kernel(const float* __restrict__ qn, const float* __restrict__ k
     float* op = o + ((size_t)r0 * H + h) * dv + col;
     const int kstep = G * dk, dstep = H * DW, vstep = H * dv;
     float sk[TC][JJ], sq[TC][JJ], sg[TC][JJ], sv[TC], sb[TC];
-    // rows beyond dk are filled with k = q = 0 and decay 1, so the arithmetic needs no bounds
+    // Rows beyond dk are filled with k = q = 0 and decay 1, and the tokens of the last chunk beyond
+    // the sequence with k = q = v = beta = 0 and decay 1, which leave the state as it is: the
+    // arithmetic needs no bounds and no branches.  A whole chunk is loaded through pointers that
+    // step from token to token; the last, partial one with every row's place computed and clamped.
+    bool in_k[JJ];
+#pragma unroll
+    for (int jj = 0; jj < JJ; ++jj) in_k[jj] = lane + 64 * jj < dk;
+    const int jlast = dk - 1;
 #define DELTA_LOAD(T0)                                                                            \
-    _Pragma("unroll") for (int tt = 0; tt < TC; ++tt) {                                           \
-        const int at = (T0) + tt < n ? (T0) + tt : n - 1;                                         \
-        _Pragma("unroll") for (int jj = 0; jj < JJ; ++jj) {                                       \
-            const int j = lane + 64 * jj;                                                         \
-            sk[tt][jj] = j < dk ? kbase[(size_t)at * kstep + j] : 0.f;                            \
-            sq[tt][jj] = j < dk ? qbase[(size_t)at * kstep + j] : 0.f;                            \
-            sg[tt][jj] = j < dk ? dbase[(size_t)at * dstep + (DW == 1 ? 0 : j)] : 1.f;            \
+    if ((T0) + TC <= n) {                                                                         \
+        const float* kp = kbase + (size_t)(T0) * kstep;                                           \
+        const float* qp = qbase + (size_t)(T0) * kstep;                                           \
+        const float* dp = dbase + (size_t)(T0) * dstep;                                           \
+        const float* vp = vbase + (size_t)(T0) * vstep;                                           \
+        const float* bp = bbase + (size_t)(T0) * H;                                               \
+        _Pragma("unroll") for (int tt = 0; tt < TC; ++tt) {                                       \
+            _Pragma("unroll") for (int jj = 0; jj < JJ; ++jj) {                                   \
+                const int j = in_k[jj] ? lane + 64 * jj : jlast;      /* read in bounds, then choose */ \
+                const float kx = kp[j], qx = qp[j], gx = dp[DW == 1 ? 0 : j];                     \
+                sk[tt][jj] = in_k[jj] ? kx : 0.f;                                                 \
+                sq[tt][jj] = in_k[jj] ? qx : 0.f;                                                 \
+                sg[tt][jj] = in_k[jj] ? gx : 1.f;                                                 \
+            }                                                                                     \
+            sv[tt] = *vp;                                                                         \
+            sb[tt] = *bp;                                                                         \
+            kp += kstep; qp += kstep; dp += dstep; vp += vstep; bp += H;                          \
         }                                                                                         \
-        sv[tt] = vbase[(size_t)at * vstep];                                                       \
-        sb[tt] = bbase[(size_t)at * H];                                                           \
+    } else {                                                                                      \
+        _Pragma("unroll") for (int tt = 0; tt < TC; ++tt) {                                       \
+            const bool ok = (T0) + tt < n;                                                        \
+            const int at = ok ? (T0) + tt : n - 1;                                                \
+            _Pragma("unroll") for (int jj = 0; jj < JJ; ++jj) {                                   \
+                const int j = in_k[jj] ? lane + 64 * jj : jlast;                                  \
+                const bool use = ok && in_k[jj];                                                  \
+                sk[tt][jj] = use ? kbase[(size_t)at * kstep + j] : 0.f;                           \
+                sq[tt][jj] = use ? qbase[(size_t)at * kstep + j] : 0.f;                           \
+                sg[tt][jj] = use ? dbase[(size_t)at * dstep + (DW == 1 ? 0 : j)] : 1.f;           \
+            }                                                                                     \
+            sv[tt] = ok ? vbase[(size_t)at * vstep] : 0.f;                                        \
+            sb[tt] = ok ? bbase[(size_t)at * H] : 0.f;                                            \
+        }                                                                                         \
     }
 #define DELTA_STORE(BUF)                                                                          \
     _Pragma("unroll") for (int tt = 0; tt < TC; ++tt) {                                           \
@@ -288,47 +317,51 @@ delta_scan_long_kernel(const float* __restrict__ qn, const float* __restrict__ k
     DELTA_LOAD(0)
     DELTA_STORE(0)
     __syncthreads();
+    const bool writes = part == 0 && live;
     for (int t0 = 0, buf = 0; t0 < n; t0 += TC, buf ^= 1) {
         float cv[TC], cb[TC];
 #pragma unroll
         for (int tt = 0; tt < TC; ++tt) { cv[tt] = sv[tt]; cb[tt] = sb[tt]; }
         const bool more = t0 + TC < n;
-        if (more) DELTA_LOAD(t0 + TC)
+        if (more) { DELTA_LOAD(t0 + TC) }
         const float* src0 = stage + (size_t)buf * TC * 3 * DKP + part;
+        float ovs[TC];
 #pragma unroll
         for (int tt = 0; tt < TC; ++tt) {
-            if (t0 + tt < n) {
-                const float* src = src0 + tt * 3 * DKP;
-                float kc[NS], pa[NA];
+            const float* src = src0 + tt * 3 * DKP;
+            float kc[NS], pa[NA];
 #pragma unroll
-                for (int a = 0; a < NA; ++a) pa[a] = 0.f;
+            for (int a = 0; a < NA; ++a) pa[a] = 0.f;
 #pragma unroll
-                for (int ii = 0; ii < NS; ++ii) {
-                    kc[ii] = src[PARTS * ii];
-                    s[ii] *= src[2 * DKP + PARTS * ii];
-                    pa[ii % NA] = fmaf(s[ii], kc[ii], pa[ii % NA]);
-                }
-                float kv = pa[0];
-#pragma unroll
-                for (int a = 1; a < NA; ++a) kv += pa[a];
-                kv = group_sum<PARTS>(kv);
-                const float u = cb[tt] * (cv[tt] - kv);
-#pragma unroll
-                for (int a = 0; a < NA; ++a) pa[a] = 0.f;
-#pragma unroll
-                for (int ii = 0; ii < NS; ++ii) {
-                    s[ii] = fmaf(kc[ii], u, s[ii]);
-                    pa[ii % NA] = fmaf(s[ii], src[DKP + PARTS * ii], pa[ii % NA]);
-                }
-                float ov = pa[0];
-#pragma unroll
-                for (int a = 1; a < NA; ++a) ov += pa[a];
-                ov = group_sum<PARTS>(ov);
-                if (part == 0 && live) *op = ov;
-                op += vstep;
+            for (int ii = 0; ii < NS; ++ii) {
+                kc[ii] = src[PARTS * ii];
+                s[ii] *= src[2 * DKP + PARTS * ii];
+                pa[ii % NA] = fmaf(s[ii], kc[ii], pa[ii % NA]);
             }
+            float kv = pa[0];
+#pragma unroll
+            for (int a = 1; a < NA; ++a) kv += pa[a];
+            kv = group_sum<PARTS>(kv);
+            const float u = cb[tt] * (cv[tt] - kv);
+#pragma unroll
+            for (int a = 0; a < NA; ++a) pa[a] = 0.f;
+#pragma unroll
+            for (int ii = 0; ii < NS; ++ii) {
+                s[ii] = fmaf(kc[ii], u, s[ii]);
+                pa[ii % NA] = fmaf(s[ii], src[DKP + PARTS * ii], pa[ii % NA]);
+            }
+            float ov = pa[0];
+#pragma unroll
+            for (int a = 1; a < NA; ++a) ov += pa[a];
+            ovs[tt] = group_sum<PARTS>(ov);
         }
-        if (more) DELTA_STORE(buf ^ 1)
+        if (writes) {
+#pragma unroll
+            for (int tt = 0; tt < TC; ++tt)
+                if (t0 + tt < n) op[(size_t)tt * vstep] = ovs[tt];
+        }
+        op += (size_t)TC * vstep;
+        if (more) { DELTA_STORE(buf ^ 1) }
         __syncthreads();
     }
 #undef DELTA_LOAD
