@@ -136,6 +136,21 @@ def test_token_by_token_and_portions_equal_the_whole_prompt(tmp_path_factory, cu
     eng.cache.check()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_portions_with_keys_and_values_of_one_width(tmp_path_factory, dtype):
+    """ODD's attention has keys and values of one width: in bfloat16 its prompts, portions (over
+    the paged cache) and single tokens run the shared matrix-core kernels with the cap."""
+    d = write_model(tmp_path_factory.getbasetemp(), ODD, seed=21, dtype=STORE[dtype])
+    w = weights64(d)
+    eng = engine_for(d, dtype)
+    ids = random_ids(150, ODD["vocab"], 29)
+    slot = eng.alloc_slot()
+    close(feed(eng, slot, ids, [40, 42, 43, 128, 140]), P.forward(ODD, w, ids), dtype, "",
+          P.decided_rows(ODD, w, ids))
+    eng.free_slot(slot)
+    eng.cache.check()
+
+
 @pytest.mark.parametrize("dtype", ["float32"])
 def test_mixed_steps_of_portions_starts_and_single_tokens(tmp_path_factory, dtype):
     """Steps that hold a sequence that starts, one that goes on by a portion and one that goes on
