@@ -333,6 +333,24 @@ def test_the_command_line_and_the_trace_replay(tmp_path):
     close(got[2], torch.stack([wa[69], wb[4]]), "float32")
 
 
+def test_a_conversation_in_one_slot(tmp_path):
+    """`Engine.session`: the turns of a conversation go on from what the slot holds (keys and
+    values, states, the convolutions' tails) by several tokens; a model with states is decoded in
+    step, so no token is ever taken back."""
+    d = write_model(tmp_path, MIXED, seed=17)
+    w = weights64(d)
+    eng = engine_for(d, "float32")
+    first = random_ids(6, MIXED["vocab"], 54)
+    with eng.session(stop_token_ids=[]) as chat:
+        a1 = chat.say(first, max_new_tokens=4)
+        assert a1 == P.greedy(MIXED, w, first, 4)
+        turn = random_ids(5, MIXED["vocab"], 77)
+        a2 = chat.say(turn, max_new_tokens=3)
+        # the token that max_new_tokens cut off is fed in front of the next turn
+        assert a2 == P.greedy(MIXED, w, first + a1 + turn, 3)
+    eng.cache.check()
+
+
 # ------------------------------------------------------------------ kernels alone
 def test_stream_mix_norm_against_plain_torch():
     from inferllm_amd.kernels import ops
