@@ -21,9 +21,9 @@ class GatedDeltaRule(Mixer):
         S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
         out  = W_o (o / rms(o) * norm * gate)
 
-    conv is a causal convolution over time per channel with `conv` taps (no bias, zeros before
-    the sequence's start); unit(x) = x / sqrt(sum x^2 + 1e-6); rms over a head's value dims with
-    `eps`.  Head h reads q/k head h / (num_heads / num_kv_heads).  `decay` "head": one g a head,
+    conv filters every channel over time with `conv` taps of its own, the last tap on the token
+    itself and nothing but zeros ahead of the sequence's first token; unit(x) = x / sqrt(sum x^2 +
+    1e-6); rms is taken over a head's value dims with `eps`.  Head h reads q/k head h / (num_heads / num_kv_heads).  `decay` "head": one g a head,
     "channel": one a head and key channel, acting on the rows of S.  Its pre-activation a is W_a h,
     or with `decay_rank` > 0 the low-rank W_a2 (W_a1 h).  `gate` "silu" or "sigmoid" of W_g h, or
     with `gate_rank` > 0 of W_g2 (W_g1 h), per head and value dim.

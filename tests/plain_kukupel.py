@@ -2,7 +2,8 @@
 the CPU, token by token where the design is recurrent.  It shares no code with the library; the
 tests compare the engine with it.
 
-Notation: h is a sublayer's input [T, E]; weights are stored [out, in] and applied as W h.
+Notation: h holds a sublayer's input rows [T, E]; a matrix W [out, in] acts on a row as W h,
+which for all rows at once is h @ W.T.
 """
 from __future__ import annotations
 
