@@ -30,6 +30,17 @@ __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf
 // `update_tail`: every sequence brings one row, and the lane that has read a channel's taps also
 // writes its tail for the next step (no other row reads that tail in this step).
 #define DELTA_VEC_MAX 4                                 // channels a lane holds: head sizes up to 256
+template <int DT>
+__device__ __forceinline__ float ld_t(const void* p, size_t i) {
+    return DT == ILLM_BF16 ? bf16_to_f32(((const bf16_t*)p)[i]) : ((const float*)p)[i];
+}
+template <int DT>
+__device__ __forceinline__ void st_t(void* p, size_t i, float v) {
+    if (DT == ILLM_BF16) ((bf16_t*)p)[i] = f32_to_bf16(v);
+    else ((float*)p)[i] = v;
+}
+
+template <int DT>                                       // the storage type of P, A and the tail
 __global__ void __launch_bounds__(256)
 delta_prepare_kernel(const void* __restrict__ P, int p_dt, int p_stride, int b_off,
                      const void* __restrict__ A, int a_dt, int a_stride, int a_off,
@@ -58,13 +69,25 @@ delta_prepare_kernel(const void* __restrict__ P, int p_dt, int p_stride, int b_o
             y[e] = 0.f;
             if (i < L) {
                 const int c = c0 + i;
-                float a = 0.f, x = 0.f;
-                for (int j = 0; j < taps; ++j) {
-                    const int d = K - j;                // tap j looks d tokens back
-                    if (d <= before) x = ld_f(P, p_dt, (size_t)(r - d) * p_stride + c);
-                    else x = ld_f(tail, tail_dt, ((size_t)slot * K + (K - (d - before))) * C + c);
-                    a = fmaf(conv_w[(size_t)c * taps + j], x, a);
-                    if (update_tail && j > 0) st_f(tail, tail_dt, ((size_t)slot * K + (j - 1)) * C + c, x);
+                // every tap's input and weight is asked for before the first is used
+                float x[DELTA_MAX_TAPS], cw[DELTA_MAX_TAPS];
+#pragma unroll
+                for (int j = 0; j < DELTA_MAX_TAPS; ++j) {
+                    x[j] = cw[j] = 0.f;
+                    if (j < taps) {
+                        const int d = K - j;            // tap j looks d tokens back
+                        x[j] = d <= before ? ld_t<DT>(P, (size_t)(r - d) * p_stride + c)
+                                           : ld_t<DT>(tail, ((size_t)slot * K + (K - (d - before))) * C + c);
+                        cw[j] = conv_w[(size_t)c * taps + j];
+                    }
+                }
+                float a = 0.f;
+#pragma unroll
+                for (int j = 0; j < DELTA_MAX_TAPS; ++j) {
+                    if (j < taps) {
+                        a = fmaf(cw[j], x[j], a);
+                        if (update_tail && j > 0) st_t<DT>(tail, ((size_t)slot * K + (j - 1)) * C + c, x[j]);
+                    }
                 }
                 y[e] = a * sigmoid_f(a);
                 ss += y[e] * y[e];
@@ -79,10 +102,10 @@ delta_prepare_kernel(const void* __restrict__ P, int p_dt, int p_stride, int b_o
             if (lane + 64 * e < L) dst[lane + 64 * e] = y[e] * inv;
     }
     for (int i = blockIdx.y * 256 + tid; i < H; i += 256 * NB)
-        beta[(size_t)r * H + i] = sigmoid_f(ld_f(P, p_dt, (size_t)r * p_stride + b_off + i));
+        beta[(size_t)r * H + i] = sigmoid_f(ld_t<DT>(P, (size_t)r * p_stride + b_off + i));
     for (int i = blockIdx.y * 256 + tid; i < H * DW; i += 256 * NB) {
         const int hh = i / DW;
-        const float a = ld_f(A, a_dt, (size_t)r * a_stride + a_off + i) + dt_bias[i];
+        const float a = ld_t<DT>(A, (size_t)r * a_stride + a_off + i) + dt_bias[i];
         dec[(size_t)r * H * DW + i] = expf(-expf(a_log[hh]) * softplus_f(a));
     }
 }
@@ -95,17 +118,20 @@ extern "C" int illm_delta_prepare(const void* P, int p_dt, int p_stride, int b_o
                                   int dv, int DW, int update_tail, void* stream) {
     if (T < 0 || G <= 0 || H <= 0 || H % G || dk <= 0 || dv <= 0 || (DW != 1 && DW != dk) ||
         dk > 64 * DELTA_VEC_MAX || dv > 64 * DELTA_VEC_MAX ||
-        taps < 1 || taps > DELTA_MAX_TAPS || !illm_dtype_ok(p_dt) || !illm_dtype_ok(a_dt) ||
-        !illm_dtype_ok(tail_dt))
+        taps < 1 || taps > DELTA_MAX_TAPS || !illm_dtype_ok(p_dt) || a_dt != p_dt || tail_dt != p_dt)
         return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
     // blocks a row: enough to fill the chip when the rows are few
     const int most = (2 * G + H + 3) / 4;
     int nb = T >= 2048 ? 1 : (2048 + T - 1) / T;
     nb = nb > most ? most : nb;
-    hipLaunchKernelGGL(delta_prepare_kernel, dim3(T, nb), dim3(256), 0, (hipStream_t)stream,
-                       P, p_dt, p_stride, b_off, A, a_dt, a_stride, a_off, conv_w, taps, tail, tail_dt,
-                       row_slot, a_log, dt_bias, qn, kn, vv, beta, dec, G, H, dk, dv, DW, update_tail);
+#define GO(DT_)                                                                                    \
+    hipLaunchKernelGGL(delta_prepare_kernel<DT_>, dim3(T, nb), dim3(256), 0, (hipStream_t)stream, P, p_dt, \
+                       p_stride, b_off, A, a_dt, a_stride, a_off, conv_w, taps, tail, tail_dt, row_slot, \
+                       a_log, dt_bias, qn, kn, vv, beta, dec, G, H, dk, dv, DW, update_tail)
+    if (p_dt == ILLM_BF16) GO(ILLM_BF16);
+    else GO(ILLM_F32);
+#undef GO
     return illm_launch_status();
 }
 

@@ -1515,6 +1515,7 @@ def delta_prepare(P: torch.Tensor, b_off: int, A: torch.Tensor, a_off: int, conv
           "delta_prepare: conv_w float32 [C, taps]")
     taps = conv_w.shape[1]
     _need(tail.dim() == 3 and tail.shape[1:] == (max(taps - 1, 1), C), "delta_prepare: tail [slots, taps - 1, C]")
+    _need(A.dtype == P.dtype and tail.dtype == P.dtype, "delta_prepare: P, A and the tail share one dtype")
     _need(a_log.dtype == torch.float32 and a_log.shape == (H,) and dt_bias.dtype == torch.float32
           and dt_bias.numel() == H * DW, "delta_prepare: a_log float32 [H], dt_bias float32 [H (dk)]")
     dev = P.device
